@@ -1,0 +1,317 @@
+#!/usr/bin/env python3
+"""Benchmark of the paged KV-cache hot path on one MI355X.
+
+A step is one layer of one decode step at the serving shape of BASELINE.json
+configs[1]: append one new K/V row per sequence into the page pool, then
+single-query paged attention over every cached row (split-K + merge).  Inputs are
+synthetic, seeded, and resident in HBM before the timed region starts.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2]
+
+Prints ONE JSON line: whole-job algorithmic HBM throughput (`value`, GB/s) with
+the decode kernel's roofline and a CPU baseline timed on the host cores.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+from dataclasses import dataclass, field
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "falcon-perception_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+import torch  # noqa: E402
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
+MODEL_LAYERS = 28       # Falcon Perception 0.6B (reference __init__.py:36)
+
+# name -> shape of the decode workloads of BASELINE.json (configs[0], [1], [3] decode part, [4])
+DECODE_WORKLOADS = {
+    "cfg1": dict(seed=1, dtype="f32", B=4, Hq=8, Hc=8, D=64, P=64, n_pages=64, prefix=0, lo=64, hi=512),
+    "cfg2": dict(seed=2, dtype="bf16", B=64, Hq=16, Hc=8, D=128, P=128, n_pages=4096, prefix=1024, lo=64, hi=3072),
+    "cfg2x": dict(seed=2, dtype="bf16", B=64, Hq=16, Hc=16, D=128, P=128, n_pages=4096, prefix=1024, lo=64, hi=3072),
+    "cfg4d": dict(seed=4, dtype="bf16", B=32, Hq=16, Hc=8, D=128, P=64, n_pages=8192, prefix=0, lo=512, hi=8192),
+    "cfg5": dict(seed=5, dtype="bf16", B=256, Hq=32, Hc=8, D=128, P=128, n_pages=None, prefix=4096, lo=256, hi=12288),
+}
+DTYPES = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
+
+
+@dataclass
+class DecodeCase:
+    """One decode step's operands, all on the device."""
+
+    name: str
+    cfg: dict
+    cache: object
+    lens: list            # context length of each sequence before the step
+    batch_idx: torch.Tensor
+    input_pos: torch.Tensor   # [B] int32 position of the new token (= lens)
+    q: torch.Tensor
+    k_new: torch.Tensor
+    v_new: torch.Tensor
+    max_context: int
+    split_tokens: int = 0
+    workspace: torch.Tensor | None = None
+    out: torch.Tensor | None = None
+    lse: torch.Tensor | None = None
+    extra: dict = field(default_factory=dict)
+
+    @property
+    def page_size(self):
+        return self.cache.page_size
+
+    @property
+    def page_table(self):
+        return self.cache.page_table
+
+    @property
+    def pool_k(self):
+        return self.cache.kv_cache[0, 0, 0]
+
+    @property
+    def pool_v(self):
+        return self.cache.kv_cache[0, 1, 0]
+
+    def append(self):
+        from falcon_perception_amd import ops
+
+        ops.kv_append(self.pool_k, self.pool_v, self.k_new, self.v_new, self.cache.page_table,
+                      self.batch_idx, self.input_pos.view(-1, 1), self.page_size, clamp_negative=True)
+
+    def attend(self):
+        from falcon_perception_amd import ops
+
+        return ops.paged_decode(self.q, self.pool_k, self.pool_v, self.cache.page_table, self.batch_idx,
+                                self.input_pos, self.page_size, self.max_context,
+                                split_tokens=self.split_tokens, workspace=self.workspace,
+                                out=self.out, lse=self.lse)
+
+    def run(self):
+        self.append()
+        return self.attend()
+
+    # ---- algorithmic traffic (bytes) --------------------------------------
+    def bytes_append(self):
+        c = self.cfg
+        e = self.q.element_size()
+        T = c["B"]
+        return 2 * T * (2 * c["Hc"] * c["D"] * e) + 8 * T
+
+    def bytes_decode(self):
+        c = self.cfg
+        e = self.q.element_size()
+        ctx = [L + 1 for L in self.lens]  # the new token attends to itself
+        return (sum(ctx) * 2 * c["Hc"] * c["D"] * e + 2 * c["B"] * c["Hq"] * c["D"] * e + 4 * c["B"] * c["Hq"]
+                + 8 * sum(math.ceil(x / c["P"]) for x in ctx))
+
+
+def make_decode_case(name: str, device="cuda", hbm_budget_gb: float | None = None) -> DecodeCase:
+    """Seeded decode workload: a fragmented page table built through the public allocator,
+    pool, q and the new K/V rows drawn from N(0,1)."""
+    from falcon_perception_amd import ops
+    from falcon_perception_amd.paged_attention import PagedKVCache
+
+    c = dict(DECODE_WORKLOADS[name])
+    dtype = DTYPES[c["dtype"]]
+    gen = torch.Generator().manual_seed(c["seed"])
+    B, P = c["B"], c["P"]
+    lens = [c["prefix"] + int(x) for x in torch.randint(c["lo"], c["hi"] + 1, (B,), generator=gen)]
+    need_pages = sum(math.ceil((L + 1) / P) for L in lens) + 1
+    n_pages = c["n_pages"]
+    if n_pages is None:  # cfg5: pool sized to ~180 GB, or to what this GPU can hold
+        e = torch.empty((), dtype=dtype).element_size()
+        page_bytes = 2 * c["Hc"] * P * c["D"] * e
+        budget = (hbm_budget_gb or 180.0) * 1e9
+        n_pages = max(need_pages, int(budget // page_bytes))
+    assert need_pages <= n_pages, f"{name}: {need_pages} pages needed, pool has {n_pages}"
+    c["n_pages"] = n_pages
+    cache = PagedKVCache(n_pages, P, B + 1, c["Hc"], c["D"], 1, dtype, device=device)
+    perm = (torch.randperm(n_pages - 1, generator=gen) + 1).tolist()
+    cache.free_pages = perm
+    slots = []
+    for L in lens:
+        b = cache.allocate()
+        cache.reserve(b, torch.tensor([b], device=device), L + 1)
+        slots.append(b)
+    dgen = torch.Generator(device=device).manual_seed(c["seed"])
+    flat = cache.kv_cache.view(-1)
+    step = 1 << 28
+    for s in range(0, flat.numel(), step):  # N(0,1) in place, chunked: no second copy of a 180 GB pool
+        flat[s:s + step].normal_(generator=dgen)
+    q = torch.randn((B, c["Hq"], 1, c["D"]), generator=dgen, device=device, dtype=torch.float32).to(dtype)
+    k_new = torch.randn((B, c["Hc"], 1, c["D"]), generator=dgen, device=device, dtype=torch.float32).to(dtype)
+    v_new = torch.randn((B, c["Hc"], 1, c["D"]), generator=dgen, device=device, dtype=torch.float32).to(dtype)
+    max_context = min(n_pages * P, math.ceil((max(lens) + 1) / P) * P)
+    case = DecodeCase(name, c, cache, lens, torch.tensor(slots, dtype=torch.int64, device=device),
+                      torch.tensor(lens, dtype=torch.int32, device=device), q, k_new, v_new, max_context)
+    case.split_tokens = ops.decode_split_tokens(B, c["Hc"], max_context, P)
+    need = ops.decode_workspace_bytes(B, c["Hq"], c["D"], max_context, case.split_tokens)
+    case.workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=device)
+    case.out = torch.empty_like(q)
+    case.lse = torch.empty((B, c["Hq"], 1), dtype=torch.float32, device=device)
+    return case
+
+
+# --------------------------------------------------------------------------
+# timing
+# --------------------------------------------------------------------------
+
+def time_steps(fn, steps: int, warmup: int) -> float:
+    """Wall-clock ms per step of `fn`, launches back to back, synchronised on both sides."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def event_ms(fn, steps: int) -> float:
+    """Average device ms per call of `fn`, HIP events on the stream the kernels run on."""
+    stream = torch.cuda.current_stream()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    for i in range(steps):
+        starts[i].record(stream)
+        fn()
+        ends[i].record(stream)
+    torch.cuda.synchronize()
+    return sum(s.elapsed_time(e) for s, e in zip(starts, ends)) / steps
+
+
+def graph_ms(fn, steps: int) -> float:
+    """ms per step when the step is replayed from a captured HIP graph (how the engine runs decode)."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fn()
+    torch.cuda.current_stream().wait_stream(side)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        fn()
+    g.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        g.replay()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def cpu_baseline(case: DecodeCase, budget_s: float = 20.0) -> dict:
+    """The reference's op sequence for one decode layer-step, ported to torch-CPU, timed on the
+    host cores on a batch subset sized to roughly `budget_s` seconds."""
+    from oracle import cpu_path
+
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    c = case.cfg
+    n = min(c["B"], 4)
+    kv = case.cache.kv_cache.cpu().float()  # upcast once, outside the timed region
+    pt = case.cache.page_table.cpu()
+    p2l = case.cache.physical_to_logical.cpu()
+
+    def one(nb):
+        sl = slice(0, nb)
+        return cpu_path.decode_step_cpu(kv, 0, pt, p2l, case.batch_idx[sl].cpu(), case.input_pos[sl].cpu(),
+                                        case.k_new[sl].cpu().float(), case.v_new[sl].cpu().float(), case.q[sl].cpu().float(),
+                                        case.page_size)
+
+    t0 = time.perf_counter()
+    one(n)
+    probe = time.perf_counter() - t0
+    per_seq = probe / n
+    nb = int(max(1, min(c["B"], (budget_s / 3) / max(per_seq, 1e-6))))
+    reps, total = 0, 0.0
+    while reps < 3 and total < budget_s:
+        t0 = time.perf_counter()
+        one(nb)
+        total += time.perf_counter() - t0
+        reps += 1
+    sec = total / reps
+    ctx = [L + 1 for L in case.lens[:nb]]
+    e = case.q.element_size()
+    alg = (sum(ctx) * 2 * c["Hc"] * c["D"] * e + 2 * nb * c["Hq"] * c["D"] * e + 4 * nb * c["Hq"]
+           + 8 * sum(math.ceil(x / c["P"]) for x in ctx) + 2 * nb * 2 * c["Hc"] * c["D"] * e + 8 * nb)
+    return {
+        "value": alg / sec / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
+        "sample": f"{nb} of {c['B']} sequences of {case.name}, {reps} repetitions, one layer-step each "
+                  f"(append + block-id gather + dense masked attention over the whole pool, fp32)",
+        "decode_tok_s_per_layer": nb / sec, "ms_per_step_sample": sec * 1e3,
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="cfg2", choices=sorted(DECODE_WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--hbm-budget-gb", type=float, default=None, help="pool size for cfg5")
+    args = ap.parse_args()
+
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU; each GPU would own its own pool, page table and "
+              "sequences with no exchange, so there is nothing to measure at N > 1.", file=sys.stderr)
+        return 2
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the hot path has no CPU implementation.", file=sys.stderr)
+        return 1
+
+    from falcon_perception_amd import _native
+
+    _native.lib()  # fail loudly if the HIP library is not built
+    case = make_decode_case(args.workload, hbm_budget_gb=args.hbm_budget_gb)
+    c = case.cfg
+
+    ms_step = time_steps(case.run, args.steps, args.warmup)
+    ms_graph = graph_ms(case.run, args.steps)
+    ms_decode = event_ms(case.attend, args.steps)
+    ms_append = event_ms(case.append, args.steps)
+
+    alg_decode = case.bytes_decode()
+    alg_append = case.bytes_append()
+    alg_step = alg_decode + alg_append
+    value = alg_step / (ms_step * 1e-3) / 1e9
+    achieved = alg_decode / (ms_decode * 1e-3) / 1e9
+
+    result = {
+        "metric": "paged decode attn + KV append HBM GB/s (% of peak); decode tok/s",
+        "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": c["dtype"], "data": "synthetic",
+        "config": {"workload": f"{case.name}: decode layer-step, batch {c['B']}, {c['Hq']} q / {c['Hc']} kv heads, "
+                               f"head_dim {c['D']}, page_size {c['P']}, {c['n_pages']}-page pool, contexts "
+                               f"{c['prefix']}+U[{c['lo']},{c['hi']}], seed {c['seed']}",
+                   "tokens_in_cache": sum(case.lens), "split_tokens": case.split_tokens},
+        "pct_of_hbm_peak": 100.0 * value / HBM_PEAK_GBPS,
+        "decode_tok_s_per_layer": c["B"] / (ms_step * 1e-3),
+        "decode_tok_s_model": c["B"] / (ms_step * 1e-3) / MODEL_LAYERS,
+        "ms_per_step_hip_graph": ms_graph,
+        "value_hip_graph": alg_step / (ms_graph * 1e-3) / 1e9,
+        "kernels": {"paged_decode_ms": ms_decode, "kv_append_ms": ms_append,
+                    "kv_append_gbps": alg_append / (ms_append * 1e-3) / 1e9},
+        "roofline": {"bound": "hbm", "kernel": "paged_decode_kernel (+ merge)", "achieved": achieved,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+                     "algorithmic_bytes": alg_decode},
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(case)
+        result["gpu_over_cpu"] = value / result["cpu_baseline"]["value"]
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

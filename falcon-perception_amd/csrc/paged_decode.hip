@@ -1,0 +1,483 @@
+// Split-K paged decode attention (one query token per sequence) and its merge.
+//
+// Replaces the reference's compiled_flex_attn_decode call (attention.py:17,
+// model.py:156-162) on the pool views that PagedKVCache.assign returns
+// (paged_attention.py:232), and the block-mask conversion that call depends on
+// (paged_attention.py:234-333, paged_inference.py:783-826): the kernel reads
+// page_table[batch_idx[b], t / P] itself and bounds the context by input_pos[b].
+//
+// HBM-bound: every cached K and V row of every sequence is read exactly once.
+//   grid  = (splits, cache heads, batch); a workgroup of 4 wavefronts owns one
+//           (sequence, cache head, token range) and serves all G = Hq / Hc query
+//           heads of that cache head from a single read of K and V.
+//   loads = a row (D elements) is covered by TPR = D * elem / 16 lanes holding
+//           16 bytes each, so a wavefront load instruction moves 64 / TPR whole
+//           rows, contiguous inside a page; U such loads of K and of V are in
+//           flight per lane before the arithmetic starts.
+//   math  = each lane group keeps its own online-softmax state (m, l, acc) in
+//           log2 space; q.k partial sums are combined across the TPR lanes with
+//           DPP adds; lane groups, then wavefronts (through LDS), then splits
+//           (through the workspace, by the merge kernel) are combined at the end.
+#include "fp_common.h"
+
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
+#include <math.h>
+
+namespace {
+
+constexpr int kWaves = 4;
+constexpr int kThreads = kWaves * 64;
+constexpr int kMaxSplitPages = 1024;  // page ids of one split held in LDS
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+struct DecodeArgs {
+  const char* q;
+  int64_t qs_b, qs_h;  // bytes
+  const char* pool_k;
+  const char* pool_v;
+  const int64_t* page_table;
+  int64_t pt_row_stride;
+  const int64_t* batch_idx;
+  const void* input_pos;
+  int pos_i64;
+  char* out;
+  int64_t os_b, os_h;  // bytes
+  float* lse;
+  float* ws_acc;  // [B, Hq, n_splits, D]
+  float* ws_ml;   // [B, Hq, n_splits, 2]
+  int Hq, Hc;
+  fp::PageDiv pd;
+  int n_pages, max_batch;
+  int64_t n_slots;
+  int max_context;
+  int split_tokens;
+  int n_splits;
+  float qscale;  // scale * log2(e)
+};
+
+// ---- element access: 16 bytes of a row as floats -------------------------
+struct F32 {
+  using type = float;
+  static constexpr int kEpl = 4;
+  static __device__ __forceinline__ void unpack(const uint4& r, float* f) {
+    f[0] = __uint_as_float(r.x);
+    f[1] = __uint_as_float(r.y);
+    f[2] = __uint_as_float(r.z);
+    f[3] = __uint_as_float(r.w);
+  }
+  static __device__ __forceinline__ void store(char* p, float v) { *reinterpret_cast<float*>(p) = v; }
+};
+struct BF16 {
+  using type = __hip_bfloat16;
+  static constexpr int kEpl = 8;
+  static __device__ __forceinline__ void unpack(const uint4& r, float* f) {
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = __uint_as_float(w[i] << 16);
+      f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+  }
+  static __device__ __forceinline__ void store(char* p, float v) {
+    *reinterpret_cast<__hip_bfloat16*>(p) = __float2bfloat16(v);
+  }
+};
+struct F16 {
+  using type = __half;
+  static constexpr int kEpl = 8;
+  static __device__ __forceinline__ void unpack(const uint4& r, float* f) {
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const __half2 h = *reinterpret_cast<const __half2*>(&w[i]);
+      const float2 x = __half22float2(h);
+      f[2 * i] = x.x;
+      f[2 * i + 1] = x.y;
+    }
+  }
+  static __device__ __forceinline__ void store(char* p, float v) { *reinterpret_cast<__half*>(p) = __float2half(v); }
+};
+
+// ---- cross-lane helpers ---------------------------------------------------
+template <int kCtrl>
+__device__ __forceinline__ float dpp(float x) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), kCtrl, 0xf, 0xf, true));
+}
+
+// sum over the kLanes consecutive lanes that share a row; every lane gets the total
+template <int kLanes>
+__device__ __forceinline__ float row_sum(float x) {
+  if (kLanes >= 2) x += dpp<0xB1>(x);   // quad_perm [1,0,3,2]
+  if (kLanes >= 4) x += dpp<0x4E>(x);   // quad_perm [2,3,0,1]
+  if (kLanes >= 8) x += dpp<0x141>(x);  // row_half_mirror
+  if (kLanes >= 16) x += dpp<0x140>(x); // row_mirror
+  if (kLanes >= 32) x += __shfl_xor(x, 16);
+  if (kLanes >= 64) x += __shfl_xor(x, 32);
+  return x;
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float safe_max(float m) { return m == -INFINITY ? 0.f : m; }
+
+// ---- main kernel ------------------------------------------------------------
+template <typename E, int D, int G, bool kDirect>
+__global__ __launch_bounds__(kThreads) void paged_decode_kernel(const DecodeArgs a) {
+  constexpr int EPL = E::kEpl;          // elements per lane
+  constexpr int TPR = D / EPL;          // lanes per row
+  constexpr int RPW = 64 / TPR;         // rows per wavefront load
+  constexpr int U = 8;                  // loads of K (and of V) in flight per lane
+  constexpr int CH = RPW * U;           // rows per wavefront iteration
+  constexpr int ROWB = D * sizeof(typename E::type);
+
+  __shared__ int s_pages[kMaxSplitPages];
+  __shared__ float s_acc[kWaves][G][D];
+  __shared__ float s_ml[kWaves][G][2];
+
+  const int split = blockIdx.x;
+  const int hc = blockIdx.y;
+  const int b = blockIdx.z;
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int lane = tid & 63;
+  const int grp = lane / TPR;  // row of this lane inside a wavefront load
+  const int col = lane % TPR;  // 16-byte chunk of the row
+
+  int64_t L = fp::load_index(a.input_pos, b, a.pos_i64) + 1;
+  const int64_t trow = a.batch_idx[b];
+  if (trow < 0 || trow >= a.max_batch) L = 0;
+  if (L > a.max_context) L = a.max_context;
+  const int t0 = split * a.split_tokens;
+  if (t0 >= L) {
+    if (kDirect && split == 0) {
+      // no visible key at all: out = 0, lse = -inf
+      for (int i = tid; i < G * D; i += kThreads) {
+        const int g = i / D, d = i - g * D;
+        E::store(a.out + b * a.os_b + (hc * G + g) * a.os_h + d * sizeof(typename E::type), 0.f);
+      }
+      if (tid < G) a.lse[static_cast<int64_t>(b) * a.Hq + hc * G + tid] = -INFINITY;
+    }
+    return;
+  }
+  const int t1 = static_cast<int>(L < t0 + a.split_tokens ? L : t0 + a.split_tokens);
+
+  // page ids of this split -> LDS
+  int64_t blk0;
+  {
+    int off_unused;
+    a.pd.split(t0, blk0, off_unused);
+    int64_t blk_last;
+    a.pd.split(t1 - 1, blk_last, off_unused);
+    const int nblk = static_cast<int>(blk_last - blk0) + 1;
+    for (int i = tid; i < nblk; i += kThreads) {
+      int64_t page = 0;
+      if (blk0 + i < a.n_pages) page = a.page_table[trow * a.pt_row_stride + blk0 + i];
+      if (page < 0 || page >= a.n_pages) page = 0;
+      s_pages[i] = static_cast<int>(page);
+    }
+  }
+
+  // query chunk of every head of the group, pre-scaled into log2 space
+  float qf[G][EPL];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    const uint4 r = *reinterpret_cast<const uint4*>(a.q + b * a.qs_b + (hc * G + g) * a.qs_h + col * 16);
+    E::unpack(r, qf[g]);
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) qf[g][e] *= a.qscale;
+  }
+
+  float m[G], l[G], acc[G][EPL];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    m[g] = -INFINITY;
+    l[g] = 0.f;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) acc[g][e] = 0.f;
+  }
+
+  const char* kbase = a.pool_k + static_cast<int64_t>(hc) * a.n_slots * ROWB + col * 16;
+  const char* vbase = a.pool_v + static_cast<int64_t>(hc) * a.n_slots * ROWB + col * 16;
+
+  __syncthreads();
+
+  for (int c0 = t0 + wave * CH; c0 < t1; c0 += kWaves * CH) {
+    uint4 kreg[U], vreg[U];
+    bool valid[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      int t = c0 + u * RPW + grp;
+      valid[u] = t < t1;
+      if (!valid[u]) t = t1 - 1;
+      int64_t blk;
+      int off;
+      a.pd.split(t, blk, off);
+      const int64_t slot = static_cast<int64_t>(s_pages[blk - blk0]) * a.pd.page_size + off;
+      kreg[u] = *reinterpret_cast<const uint4*>(kbase + slot * ROWB);
+      vreg[u] = *reinterpret_cast<const uint4*>(vbase + slot * ROWB);
+    }
+
+    float s[G][U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      float kf[EPL];
+      E::unpack(kreg[u], kf);
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        float p = 0.f;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) p = fmaf(qf[g][e], kf[e], p);
+        s[g][u] = p;
+      }
+    }
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const float tot = row_sum<TPR>(s[g][u]);
+        s[g][u] = valid[u] ? tot : -INFINITY;
+      }
+    }
+
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      float mx = m[g];
+#pragma unroll
+      for (int u = 0; u < U; ++u) mx = fmaxf(mx, s[g][u]);
+      const float ms = safe_max(mx);
+      const float alpha = fast_exp2(m[g] - ms);
+      m[g] = mx;
+      float ps = 0.f;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        s[g][u] = fast_exp2(s[g][u] - ms);
+        ps += s[g][u];
+      }
+      l[g] = l[g] * alpha + ps;
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) acc[g][e] *= alpha;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      float vf[EPL];
+      E::unpack(vreg[u], vf);
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) acc[g][e] = fmaf(s[g][u], vf[e], acc[g][e]);
+      }
+    }
+  }
+
+  // combine the lane groups of this wavefront
+#pragma unroll
+  for (int off = TPR; off < 64; off <<= 1) {
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const float mo = __shfl_xor(m[g], off);
+      const float lo = __shfl_xor(l[g], off);
+      const float mn = fmaxf(m[g], mo);
+      const float ms = safe_max(mn);
+      const float wa = fast_exp2(m[g] - ms);
+      const float wb = fast_exp2(mo - ms);
+      l[g] = l[g] * wa + lo * wb;
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) acc[g][e] = acc[g][e] * wa + __shfl_xor(acc[g][e], off) * wb;
+      m[g] = mn;
+    }
+  }
+  if (lane < TPR) {
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) s_acc[wave][g][col * EPL + e] = acc[g][e];
+      if (lane == 0) {
+        s_ml[wave][g][0] = m[g];
+        s_ml[wave][g][1] = l[g];
+      }
+    }
+  }
+  __syncthreads();
+
+  // combine the wavefronts; one thread per (head of the group, element)
+  for (int i = tid; i < G * D; i += kThreads) {
+    const int g = i / D, d = i - g * D;
+    float mn = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) mn = fmaxf(mn, s_ml[w][g][0]);
+    const float ms = safe_max(mn);
+    float num = 0.f, den = 0.f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      const float wgt = fast_exp2(s_ml[w][g][0] - ms);
+      num += s_acc[w][g][d] * wgt;
+      den += s_ml[w][g][1] * wgt;
+    }
+    const int hq = hc * G + g;
+    if (kDirect) {
+      E::store(a.out + b * a.os_b + hq * a.os_h + d * sizeof(typename E::type), num / den);
+      if (d == 0) a.lse[static_cast<int64_t>(b) * a.Hq + hq] = (mn + log2f(den)) * kLn2;
+    } else {
+      const int64_t p = (static_cast<int64_t>(b) * a.Hq + hq) * a.n_splits + split;
+      a.ws_acc[p * D + d] = num;
+      if (d == 0) {
+        a.ws_ml[p * 2] = mn;
+        a.ws_ml[p * 2 + 1] = den;
+      }
+    }
+  }
+}
+
+// ---- cross-split merge ------------------------------------------------------
+template <typename E, int D>
+__global__ __launch_bounds__(64) void paged_decode_merge_kernel(const DecodeArgs a) {
+  const int hq = blockIdx.x;
+  const int b = blockIdx.y;
+  int64_t L = fp::load_index(a.input_pos, b, a.pos_i64) + 1;
+  const int64_t trow = a.batch_idx[b];
+  if (trow < 0 || trow >= a.max_batch) L = 0;
+  if (L > a.max_context) L = a.max_context;
+  const int ns = L <= 0 ? 0 : static_cast<int>((L + a.split_tokens - 1) / a.split_tokens);
+  const int64_t p0 = (static_cast<int64_t>(b) * a.Hq + hq) * a.n_splits;
+
+  float mn = -INFINITY;
+  for (int s = 0; s < ns; ++s) mn = fmaxf(mn, a.ws_ml[(p0 + s) * 2]);
+  const float ms = safe_max(mn);
+  float den = 0.f;
+  for (int s = 0; s < ns; ++s) den += a.ws_ml[(p0 + s) * 2 + 1] * fast_exp2(a.ws_ml[(p0 + s) * 2] - ms);
+
+  for (int d = threadIdx.x; d < D; d += 64) {
+    float num = 0.f;
+    for (int s = 0; s < ns; ++s) num += a.ws_acc[(p0 + s) * D + d] * fast_exp2(a.ws_ml[(p0 + s) * 2] - ms);
+    const float o = ns > 0 ? num / den : 0.f;
+    E::store(a.out + b * a.os_b + hq * a.os_h + d * sizeof(typename E::type), o);
+  }
+  if (threadIdx.x == 0)
+    a.lse[static_cast<int64_t>(b) * a.Hq + hq] = ns > 0 ? (mn + log2f(den)) * kLn2 : -INFINITY;
+}
+
+template <typename E, int D, int G>
+void launch_decode(const DecodeArgs& a, int B, hipStream_t st) {
+  dim3 grid(a.n_splits, a.Hc, B);
+  if (a.n_splits == 1) {
+    hipLaunchKernelGGL((paged_decode_kernel<E, D, G, true>), grid, dim3(kThreads), 0, st, a);
+  } else {
+    hipLaunchKernelGGL((paged_decode_kernel<E, D, G, false>), grid, dim3(kThreads), 0, st, a);
+    hipLaunchKernelGGL((paged_decode_merge_kernel<E, D>), dim3(a.Hq, B), dim3(64), 0, st, a);
+  }
+}
+
+template <typename E, int D>
+int dispatch_group(const DecodeArgs& a, int B, hipStream_t st) {
+  switch (a.Hq / a.Hc) {
+    case 1: launch_decode<E, D, 1>(a, B, st); return FP_OK;
+    case 2: launch_decode<E, D, 2>(a, B, st); return FP_OK;
+    case 4: launch_decode<E, D, 4>(a, B, st); return FP_OK;
+    case 8: launch_decode<E, D, 8>(a, B, st); return FP_OK;
+    default: return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_decode: Hq/Hc = %d (supported: 1, 2, 4, 8)", a.Hq / a.Hc);
+  }
+}
+
+template <typename E>
+int dispatch_dim(const DecodeArgs& a, int B, int D, hipStream_t st) {
+  switch (D) {
+    case 64: return dispatch_group<E, 64>(a, B, st);
+    case 128: return dispatch_group<E, 128>(a, B, st);
+    default: return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_decode: head_dim %d (supported: 64, 128)", D);
+  }
+}
+
+int default_split_tokens(int B, int Hc, int max_context, int page_size) {
+  int split = 1024;
+  while (split > 128 && static_cast<int64_t>(B) * Hc * ((max_context + split - 1) / split) < 2048) split >>= 1;
+  while (split / page_size + 2 > kMaxSplitPages) split >>= 1;
+  return split < 64 ? 64 : split;
+}
+
+int n_splits_for(int max_context, int split_tokens) {
+  const int n = (max_context + split_tokens - 1) / split_tokens;
+  return n < 1 ? 1 : n;
+}
+
+}  // namespace
+
+extern "C" int32_t fp_paged_decode_default_split(int32_t B, int32_t Hc, int32_t max_context, int32_t page_size) {
+  if (B <= 0 || Hc <= 0 || max_context < 0 || page_size <= 0)
+    return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode_default_split: bad dimension");
+  return default_split_tokens(B, Hc, max_context, page_size);
+}
+
+extern "C" int64_t fp_paged_decode_workspace_bytes(int32_t B, int32_t Hq, int32_t D, int32_t max_context,
+                                                   int32_t split_tokens) {
+  if (B < 0 || Hq <= 0 || D <= 0 || max_context < 0 || split_tokens <= 0)
+    return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode_workspace_bytes: bad dimension");
+  if (split_tokens % 64) return fp::fail(FP_ERR_INVALID_ARGUMENT, "split_tokens must be a multiple of 64");
+  const int64_t ns = n_splits_for(max_context, split_tokens);
+  if (ns == 1) return 0;
+  return static_cast<int64_t>(B) * Hq * ns * (D + 2) * static_cast<int64_t>(sizeof(float));
+}
+
+extern "C" int fp_paged_decode(const void* q, int64_t q_stride_b, int64_t q_stride_h, const void* pool_k,
+                               const void* pool_v, const int64_t* page_table, int64_t pt_row_stride,
+                               const int64_t* batch_idx, const void* input_pos, int pos_index_type,
+                               void* out, int64_t out_stride_b, int64_t out_stride_h, float* lse,
+                               void* workspace, int64_t workspace_bytes, int32_t B, int32_t Hq, int32_t Hc,
+                               int32_t D, int32_t page_size, int32_t n_pages, int32_t max_batch,
+                               int64_t n_slots, int32_t max_context, int32_t split_tokens, float scale,
+                               int dtype, void* stream) {
+  const int eb = fp::elem_bytes(dtype);
+  if (eb == 0) return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_decode: unknown dtype %d", dtype);
+  if (B < 0 || Hq <= 0 || Hc <= 0 || D <= 0 || page_size <= 0 || n_pages <= 0 || max_batch <= 0 ||
+      n_slots <= 0 || max_context < 0 || split_tokens < 0)
+    return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: bad dimension");
+  if (Hq % Hc) return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: Hq=%d not a multiple of Hc=%d", Hq, Hc);
+  if (n_slots < static_cast<int64_t>(n_pages) * page_size)
+    return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: n_slots smaller than n_pages * page_size");
+  if (max_context > static_cast<int64_t>(n_pages) * page_size)
+    return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: max_context exceeds the page table width");
+  if (pos_index_type != FP_INDEX_I32 && pos_index_type != FP_INDEX_I64)
+    return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: bad pos_index_type");
+  if (B > 65535 || Hc > 65535 || Hq > 65535)
+    return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_decode: B, Hq or Hc exceeds 65535");
+  if (B == 0) return FP_OK;
+  if (!q || !pool_k || !pool_v || !page_table || !batch_idx || !input_pos || !out || !lse)
+    return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: null pointer");
+  if (!fp::aligned(q, 16) || !fp::aligned(pool_k, 16) || !fp::aligned(pool_v, 16) ||
+      (q_stride_b * eb) % 16 || (q_stride_h * eb) % 16)
+    return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: q and pool rows must be 16-byte aligned");
+  if (!fp::aligned(out, eb)) return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: out misaligned");
+
+  if (split_tokens == 0) split_tokens = default_split_tokens(B, Hc, max_context, page_size);
+  if (split_tokens % 64) return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: split_tokens must be a multiple of 64");
+  if (split_tokens / page_size + 2 > kMaxSplitPages)
+    return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_decode: split of %d tokens spans more than %d pages", split_tokens,
+                    kMaxSplitPages - 2);
+  const int ns = n_splits_for(max_context, split_tokens);
+  if (ns > 65535) return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_decode: more than 65535 splits");
+
+  DecodeArgs a{static_cast<const char*>(q), q_stride_b * eb, q_stride_h * eb,
+               static_cast<const char*>(pool_k), static_cast<const char*>(pool_v),
+               page_table, pt_row_stride, batch_idx, input_pos, pos_index_type == FP_INDEX_I64,
+               static_cast<char*>(out), out_stride_b * eb, out_stride_h * eb, lse,
+               nullptr, nullptr, Hq, Hc, fp::PageDiv(page_size), n_pages, max_batch, n_slots,
+               max_context, split_tokens, ns, scale * kLog2e};
+  if (ns > 1) {
+    const int64_t need = static_cast<int64_t>(B) * Hq * ns * (D + 2) * static_cast<int64_t>(sizeof(float));
+    if (!workspace || workspace_bytes < need || !fp::aligned(workspace, 16))
+      return fp::fail(FP_ERR_WORKSPACE, "fp_paged_decode: workspace of %lld bytes needed, %lld given",
+                      static_cast<long long>(need), static_cast<long long>(workspace_bytes));
+    a.ws_acc = static_cast<float*>(workspace);
+    a.ws_ml = a.ws_acc + static_cast<int64_t>(B) * Hq * ns * D;
+  }
+
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  int rc;
+  switch (dtype) {
+    case FP_DTYPE_F32: rc = dispatch_dim<F32>(a, B, D, st); break;
+    case FP_DTYPE_BF16: rc = dispatch_dim<BF16>(a, B, D, st); break;
+    default: rc = dispatch_dim<F16>(a, B, D, st); break;
+  }
+  if (rc != FP_OK) return rc;
+  return fp::check_launch("fp_paged_decode");
+}

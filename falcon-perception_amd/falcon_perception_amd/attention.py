@@ -1,0 +1,278 @@
+"""Attention entry points with the reference's names and call signature.
+
+The reference binds `compiled_flex_attn_decode` / `compiled_flex_attn_prefill`
+(`falcon_perception/attention.py:17-18`) in `model.py:20-24` and calls them as
+`fn(q, k, v, block_mask=..., return_aux=AuxRequest(lse=True), kernel_options=...)`
+(`model.py:156-162`).  Here the same names dispatch on the mask object:
+
+* a `PagedDecodeMask` (what `PagedKVCache.convert_logical_block_mask` returns) runs
+  the split-K paged decode kernel,
+* a `HybridPrefillMask` (what `PagedKVCache.create_prefill_blockmask` returns) runs
+  the MFMA chunked-prefill kernel over the paged cache,
+* any other mask is not part of the paged path (the reference's AnyUp upsampler
+  uses a windowed torch BlockMask, `anyup.py:358`) and is handed to torch's own
+  flex_attention untouched.
+
+The mask-mod factories and `create_attention_mask` keep the reference's names
+(`attention.py:22-131`) because `paged_attention.py:16-20`, `model.py:23` and
+`batch_inference.py:8` import them.
+"""
+
+from __future__ import annotations
+
+import torch
+from torch import Tensor
+from torch.nn.attention.flex_attention import AuxOutput, BlockMask, and_masks, or_masks
+
+from . import ops
+
+__all__ = [
+    "compiled_flex_attn_decode",
+    "compiled_flex_attn_prefill",
+    "create_attention_mask",
+    "create_batch_attention_mask",
+    "get_causal_mask_mod",
+    "get_document_mask_mod",
+    "get_image_prefix_mask_mod",
+    "get_non_left_pad_mask_mod",
+    "offset_mask_mod",
+    "PagedDecodeMask",
+    "HybridPrefillMask",
+]
+
+
+# --------------------------------------------------------------------------
+# mask objects of the paged path
+# --------------------------------------------------------------------------
+
+class PagedDecodeMask:
+    """Decode-step mask in physical page space.
+
+    Returned by `PagedKVCache.convert_logical_block_mask`.  The decode kernel needs
+    only the cache (page table), the batch rows and the positions of the step, so
+    the physical block lists the reference materialises every step
+    (`paged_attention.py:279-301`) are computed on first access only.
+    """
+
+    def __init__(self, cache, logical: BlockMask, batch_idx: Tensor):
+        self.cache = cache
+        self.logical = logical
+        self.batch_idx = batch_idx
+        self.BLOCK_SIZE = logical.BLOCK_SIZE
+        self.seq_lengths = (logical.seq_lengths[0], cache.n_pages * cache.page_size)
+        self._physical: dict[str, Tensor | None] = {}
+
+    @property
+    def max_context(self) -> int:
+        """Upper bound of the logical context length (KV length of the logical mask)."""
+        return min(int(self.logical.seq_lengths[1]), self.cache.n_pages * self.cache.page_size)
+
+    def _converted(self, name: str) -> Tensor | None:
+        if name not in self._physical:
+            src = getattr(self.logical, name)
+            self._physical[name] = (
+                None if src is None else ops.convert_block_ids(src, self.cache.page_table, self.batch_idx)
+            )
+        return self._physical[name]
+
+    @property
+    def kv_num_blocks(self) -> Tensor:
+        return self.logical.kv_num_blocks.clone()
+
+    @property
+    def kv_indices(self) -> Tensor:
+        return self._converted("kv_indices")
+
+    @property
+    def full_kv_num_blocks(self) -> Tensor | None:
+        src = self.logical.full_kv_num_blocks
+        return None if src is None else src.clone()
+
+    @property
+    def full_kv_indices(self) -> Tensor | None:
+        return self._converted("full_kv_indices")
+
+    @property
+    def mask_mod(self):
+        return self.cache.get_mask_mod(self.logical.mask_mod, self.batch_idx)
+
+    def as_block_mask(self) -> BlockMask:
+        """The torch BlockMask the reference would have built (`paged_attention.py:293-301`)."""
+        return BlockMask.from_kv_blocks(
+            self.kv_num_blocks, self.kv_indices, self.full_kv_num_blocks, self.full_kv_indices,
+            self.BLOCK_SIZE, self.mask_mod, seq_lengths=self.seq_lengths,
+        )
+
+
+class HybridPrefillMask:
+    """Prefill mask: document-causal OR bidirectional inside an image span.
+
+    Returned by `PagedKVCache.create_prefill_blockmask`.  Holds, per packed row, the
+    packed index one past the last key the row may see (`row_hi`); together with the
+    row's own position this is the whole mask (`attention.py:75-96`,
+    `paged_attention.py:353-359`).
+    """
+
+    def __init__(self, cache, batch_idx: Tensor, input_ids: Tensor, soi_id: int, eoi_id: int, block_size: int):
+        self.cache = cache
+        self.batch_idx = batch_idx
+        self.input_ids = input_ids
+        self.soi_id = soi_id
+        self.eoi_id = eoi_id
+        self.BLOCK_SIZE = (block_size, block_size)
+        L = batch_idx.shape[1]
+        self.seq_lengths = (L, L)
+        self.row_hi = ops.hybrid_row_limits(input_ids, soi_id, eoi_id)  # [L] int32, packed coordinates
+        self._arange = torch.arange(L, dtype=torch.int64, device=batch_idx.device)
+
+    def row_limit(self, input_pos: Tensor) -> Tensor:
+        """Logical key limit of each row: its position plus the reach of `row_hi` beyond the row."""
+        reach = self.row_hi.to(torch.int64) - self._arange
+        return (input_pos.reshape(-1) + reach).to(torch.int32)
+
+
+# --------------------------------------------------------------------------
+# the two attention callables
+# --------------------------------------------------------------------------
+
+_torch_flex = {}
+
+
+def _foreign(kind: str, q, k, v, kwargs):
+    """Masks this package does not own go to torch's flex_attention unchanged."""
+    if kind not in _torch_flex:
+        from torch.nn.attention.flex_attention import flex_attention
+
+        opts = {"fullgraph": True} if kind == "decode" else {"dynamic": True}
+        _torch_flex[kind] = torch.compile(flex_attention, **opts)
+    return _torch_flex[kind](q, k, v, **kwargs)
+
+
+def _result(out: Tensor, lse: Tensor, return_aux, return_lse: bool):
+    if return_aux is not None:
+        want_lse = getattr(return_aux, "lse", False)
+        return out, AuxOutput(lse=lse if want_lse else None)
+    if return_lse:
+        return out, lse
+    return out
+
+
+def compiled_flex_attn_decode(q: Tensor, k: Tensor, v: Tensor, score_mod=None, block_mask=None,
+                              scale: float | None = None, enable_gqa: bool = False,
+                              return_lse: bool = False, kernel_options=None, *, return_aux=None):
+    """Decode attention, one query token per sequence (`attention.py:17`, `model.py:156-162`).
+
+    q [B, Hq, 1, D]; k, v are the pool views `PagedKVCache.insert_kv` returned,
+    [1, Hc, n_slots, D].  `kernel_options` are Triton tuning knobs of the reference
+    and are ignored.
+    """
+    if not isinstance(block_mask, PagedDecodeMask):
+        return _foreign("decode", q, k, v, dict(score_mod=score_mod, block_mask=block_mask, scale=scale,
+                                                enable_gqa=enable_gqa, return_lse=return_lse,
+                                                kernel_options=kernel_options, return_aux=return_aux))
+    if score_mod is not None:
+        raise RuntimeError("score_mod is not supported on the paged decode path")
+    cache = block_mask.cache
+    step = cache.last_decode_step
+    if step is None:
+        raise RuntimeError("paged decode attention called before PagedKVCache.insert_kv for this step")
+    if q.shape[2] != 1:
+        raise RuntimeError("a PagedDecodeMask serves one query token per sequence")
+    out, lse = ops.paged_decode(
+        q, k[0], v[0], cache.page_table, block_mask.batch_idx, step.input_pos,
+        cache.page_size, block_mask.max_context, scale=scale,
+        workspace=cache.decode_workspace(q.shape[0], q.shape[1], q.shape[3], block_mask.max_context, k.shape[1]),
+        split_tokens=cache.decode_split_tokens(q.shape[0], k.shape[1], block_mask.max_context),
+    )
+    return _result(out, lse, return_aux, return_lse)
+
+
+def compiled_flex_attn_prefill(q: Tensor, k: Tensor, v: Tensor, score_mod=None, block_mask=None,
+                               scale: float | None = None, enable_gqa: bool = False,
+                               return_lse: bool = False, kernel_options=None, *, return_aux=None):
+    """Prefill attention over the paged cache under the hybrid mask (`attention.py:18`).
+
+    q [1, Hq, L, D] packed rows.  Keys and values are read from the pages that
+    `PagedKVCache.insert_kv` has just filled for this layer (the k, v arguments are
+    the fresh rows it returned and are not read again), so a chunk whose prefix
+    already lives in pages attends over prefix and chunk alike.
+    """
+    if not isinstance(block_mask, HybridPrefillMask):
+        return _foreign("prefill", q, k, v, dict(score_mod=score_mod, block_mask=block_mask, scale=scale,
+                                                 enable_gqa=enable_gqa, return_lse=return_lse,
+                                                 kernel_options=kernel_options, return_aux=return_aux))
+    if score_mod is not None:
+        raise RuntimeError("score_mod is not supported on the paged prefill path")
+    cache = block_mask.cache
+    step = cache.last_prefill_step
+    if step is None:
+        raise RuntimeError("paged prefill attention called before PagedKVCache.insert_kv for this step")
+    pool_k = cache.kv_cache[step.layer_id, 0, 0]
+    pool_v = cache.kv_cache[step.layer_id, 1, 0]
+    out, lse = ops.paged_prefill(
+        q, pool_k, pool_v, cache.page_table, step.batch_idx, step.input_pos,
+        block_mask.row_limit(step.input_pos), cache.page_size, scale=scale,
+    )
+    return _result(out, lse, return_aux, return_lse)
+
+
+# --------------------------------------------------------------------------
+# mask-mod factories (names of attention.py:22-131)
+# --------------------------------------------------------------------------
+
+def offset_mask_mod(mask_mod, offset: int):
+    """mask_mod evaluated with the query index shifted by `offset` (`attention.py:22-28`)."""
+    return lambda b, h, q, kv: mask_mod(b, h, q + offset, kv)
+
+
+def get_causal_mask_mod():
+    """kv may not lie after q (`attention.py:31-37`)."""
+    return lambda b, h, q_idx, kv_idx: q_idx >= kv_idx
+
+
+def get_document_mask_mod(batch: Tensor, eos_id: int):
+    """Tokens attend only inside their own eos-delimited document (`attention.py:40-60`)."""
+    ends = batch == eos_id
+    ends[:, -1] = True
+    closed = torch.cumsum(ends.to(torch.int32), dim=1)
+    doc_id = torch.zeros_like(closed, dtype=torch.int32)
+    doc_id[:, 1:] = closed[:, :-1]
+    return lambda b, h, q_idx, kv_idx: doc_id[b, q_idx] == doc_id[b, kv_idx]
+
+
+def get_non_left_pad_mask_mod(batch: Tensor, pad_id: int):
+    """Keys that are left padding are never attended (`attention.py:63-72`)."""
+    seen_real = torch.cumsum(batch != pad_id, dim=1)
+    return lambda b, h, q_idx, kv_idx: seen_real[b, kv_idx] > 0
+
+
+def get_image_prefix_mask_mod(batch: Tensor, soi_id: int, eoi_id: int):
+    """Bidirectional attention between tokens of one image span (`attention.py:75-96`)."""
+    opened = torch.cumsum(batch == soi_id, dim=1)
+    closed = torch.cumsum(batch == eoi_id, dim=1)
+    inside = (opened - closed) > 0
+    span = opened * inside
+    return lambda b, h, q_idx, kv_idx: (inside[b, q_idx] & inside[b, kv_idx]) & (span[b, q_idx] == span[b, kv_idx])
+
+
+@torch.inference_mode()
+def create_attention_mask(*args, **kwargs) -> BlockMask:
+    """torch `create_block_mask` under inference mode (`attention.py:99-102`).
+
+    Only masks outside the paged path are built this way (the dense batch engine);
+    the paged path builds its masks in closed form in `paged_attention.py`.
+    """
+    from torch.nn.attention.flex_attention import create_block_mask
+
+    return create_block_mask(*args, **kwargs)
+
+
+def create_batch_attention_mask(input_batch: Tensor, *, pad_token_id: int, eos_token_id: int,
+                                soi_token_id: int, eoi_token_id: int, max_len: int | None = None) -> BlockMask:
+    """Mask of the dense batch engine (`attention.py:105-131`): image-prefix OR (causal AND document AND non-left-pad)."""
+    B, S = input_batch.size()
+    text = and_masks(get_causal_mask_mod(), get_document_mask_mod(input_batch, eos_token_id),
+                     get_non_left_pad_mask_mod(input_batch, pad_token_id))
+    image = get_image_prefix_mask_mod(input_batch, soi_token_id, eoi_token_id)
+    n = max_len or S
+    return create_attention_mask(or_masks(image, text), B, None, n, n)

@@ -1,0 +1,190 @@
+"""Tensor-level wrappers of the C ABI: torch supplies device memory and the stream,
+the HIP kernels of libfp_paged_kv.so do the work.  No wrapper allocates unless the
+caller leaves an output or workspace argument out, and none synchronises.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+from torch import Tensor
+
+from . import _native as N
+
+
+def _rows(t: Tensor) -> Tensor:
+    """Make the head_dim axis dense (the kernels move whole rows)."""
+    return t if t.stride(-1) == 1 else t.contiguous()
+
+
+def kv_append(pool_k: Tensor, pool_v: Tensor, k: Tensor, v: Tensor, page_table: Tensor,
+              batch_idx: Tensor, input_pos: Tensor, page_size: int, clamp_negative: bool) -> None:
+    """Scatter k, v [T, H, S, D] into pool_k, pool_v [H, N, D] at the slots the page table gives.
+
+    batch_idx [T] int64, input_pos [T, S] int32/int64.  Byte-exact copy
+    (reference paged_attention.py:212-230 with clamp, :387-391 without).
+    """
+    N.require_cuda(pool_k, pool_v, k, v, page_table, batch_idx, input_pos)
+    T, H, S, D = k.shape
+    if v.shape != k.shape:
+        raise RuntimeError(f"k {tuple(k.shape)} and v {tuple(v.shape)} must have the same shape")
+    if pool_k.dtype != k.dtype or pool_v.dtype != v.dtype:
+        raise RuntimeError(f"dtype mismatch: pool {pool_k.dtype}, k {k.dtype}, v {v.dtype}")
+    if not (pool_k.is_contiguous() and pool_v.is_contiguous()):
+        raise RuntimeError("pool planes must be contiguous [H, N, D]")
+    k, v = _rows(k), _rows(v)
+    input_pos = input_pos.contiguous()
+    batch_idx = batch_idx.contiguous()
+    if batch_idx.dtype != torch.int64:
+        batch_idx = batch_idx.to(torch.int64)
+    if page_table.dtype != torch.int64 or page_table.stride(1) != 1:
+        raise RuntimeError("page_table must be int64 with a dense last axis")
+    Hp, n_slots, Dp = pool_k.shape
+    rc = N.lib().fp_kv_append(
+        pool_k.data_ptr(), pool_v.data_ptr(), k.data_ptr(), v.data_ptr(),
+        k.stride(0), k.stride(1), k.stride(2), v.stride(0), v.stride(1), v.stride(2),
+        page_table.data_ptr(), page_table.stride(0), batch_idx.data_ptr(),
+        input_pos.data_ptr(), N.index_code(input_pos),
+        T, H, S, D, page_size, page_table.shape[1], page_table.shape[0],
+        n_slots, N.dtype_code(k.dtype), int(clamp_negative), N.stream_ptr(k.device))
+    N.check(rc, "fp_kv_append")
+
+
+def kv_gather(pool: Tensor, page_table: Tensor, batch_idx: Tensor, seq_lens: Tensor,
+              page_size: int, max_len: int, out: Tensor | None = None) -> Tensor:
+    """Dense logical view [B, H, max_len, D] of the cached rows of each sequence; zero tail."""
+    N.require_cuda(pool, page_table, batch_idx, seq_lens, out)
+    H, n_slots, D = pool.shape
+    B = batch_idx.shape[0]
+    if out is None:
+        out = torch.empty((B, H, max_len, D), dtype=pool.dtype, device=pool.device)
+    elif out.shape != (B, H, max_len, D) or out.dtype != pool.dtype or out.stride(3) != 1:
+        raise RuntimeError("out must be [B, H, max_len, D] of the pool dtype with dense rows")
+    batch_idx = batch_idx.contiguous()
+    seq_lens = seq_lens.contiguous()
+    rc = N.lib().fp_kv_gather(
+        pool.data_ptr(), out.data_ptr(), out.stride(0), out.stride(1), out.stride(2),
+        page_table.data_ptr(), page_table.stride(0), batch_idx.data_ptr(),
+        seq_lens.data_ptr(), N.index_code(seq_lens),
+        B, H, max_len, D, page_size, page_table.shape[1], page_table.shape[0],
+        n_slots, N.dtype_code(pool.dtype), N.stream_ptr(pool.device))
+    N.check(rc, "fp_kv_gather")
+    return out
+
+
+def convert_block_ids(kv_indices: Tensor, page_table: Tensor, batch_idx: Tensor) -> Tensor:
+    """kv_indices [B, H, R, C] int32 logical blocks -> [B, H, R, n_pages] int32 physical pages."""
+    N.require_cuda(kv_indices, page_table, batch_idx)
+    B, H, R, C = kv_indices.shape
+    n_pages = page_table.shape[1]
+    if kv_indices.dtype != torch.int32:
+        kv_indices = kv_indices.to(torch.int32)
+    kv_indices = kv_indices.contiguous()
+    batch_idx = batch_idx.contiguous()
+    out = torch.empty((B, H, R, n_pages), dtype=torch.int32, device=kv_indices.device)
+    rc = N.lib().fp_convert_block_ids(
+        kv_indices.data_ptr(), out.data_ptr(), page_table.data_ptr(), page_table.stride(0),
+        batch_idx.data_ptr(), B, H * R, C, n_pages, page_table.shape[0],
+        N.stream_ptr(kv_indices.device))
+    N.check(rc, "fp_convert_block_ids")
+    return out
+
+
+def decode_split_tokens(B: int, Hc: int, max_context: int, page_size: int) -> int:
+    return int(N.lib().fp_paged_decode_default_split(B, Hc, max_context, page_size))
+
+
+def decode_workspace_bytes(B: int, Hq: int, D: int, max_context: int, split_tokens: int) -> int:
+    n = int(N.lib().fp_paged_decode_workspace_bytes(B, Hq, D, max_context, split_tokens))
+    N.check(n, "fp_paged_decode_workspace_bytes")
+    return n
+
+
+def paged_decode(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor, batch_idx: Tensor,
+                 input_pos: Tensor, page_size: int, max_context: int, *, scale: float | None = None,
+                 split_tokens: int = 0, workspace: Tensor | None = None,
+                 out: Tensor | None = None, lse: Tensor | None = None) -> tuple[Tensor, Tensor]:
+    """Single-query paged attention.  q [B, Hq, 1, D]; pools [Hc, N, D]; returns out [B, Hq, 1, D], lse [B, Hq, 1]."""
+    N.require_cuda(q, pool_k, pool_v, page_table, batch_idx, input_pos, workspace, out, lse)
+    B, Hq, Sq, D = q.shape
+    if Sq != 1:
+        raise RuntimeError(f"paged_decode takes one query token per sequence, got {Sq}")
+    Hc, n_slots, Dp = pool_k.shape
+    if Dp != D or pool_v.shape != pool_k.shape or pool_k.dtype != q.dtype or pool_v.dtype != q.dtype:
+        raise RuntimeError("q / pool shape or dtype mismatch")
+    q = _rows(q)
+    input_pos = input_pos.reshape(-1).contiguous()
+    batch_idx = batch_idx.contiguous()
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    if split_tokens == 0:
+        split_tokens = decode_split_tokens(B, Hc, max_context, page_size)
+    need = decode_workspace_bytes(B, Hq, D, max_context, split_tokens)
+    if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
+        workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+    if out is None:
+        out = torch.empty((B, Hq, 1, D), dtype=q.dtype, device=q.device)
+    if lse is None:
+        lse = torch.empty((B, Hq, 1), dtype=torch.float32, device=q.device)
+    if out.stride(3) != 1 or not lse.is_contiguous() or lse.dtype != torch.float32:
+        raise RuntimeError("out rows must be dense and lse contiguous float32")
+    rc = N.lib().fp_paged_decode(
+        q.data_ptr(), q.stride(0), q.stride(1), pool_k.data_ptr(), pool_v.data_ptr(),
+        page_table.data_ptr(), page_table.stride(0), batch_idx.data_ptr(),
+        input_pos.data_ptr(), N.index_code(input_pos),
+        out.data_ptr(), out.stride(0), out.stride(1), lse.data_ptr(),
+        workspace.data_ptr() if workspace is not None else None,
+        workspace.numel() * workspace.element_size() if workspace is not None else 0,
+        B, Hq, Hc, D, page_size, page_table.shape[1], page_table.shape[0],
+        n_slots, max_context, split_tokens, scale, N.dtype_code(q.dtype), N.stream_ptr(q.device))
+    N.check(rc, "fp_paged_decode")
+    return out, lse
+
+
+def hybrid_row_limits(input_ids: Tensor, soi_id: int, eoi_id: int) -> Tensor:
+    """Packed index one past the last key each packed row may see: max(q + 1, end of q's image span)."""
+    N.require_cuda(input_ids)
+    ids = input_ids.reshape(-1).contiguous()
+    if ids.dtype != torch.int64:
+        ids = ids.to(torch.int64)
+    out = torch.empty(ids.shape[0], dtype=torch.int32, device=ids.device)
+    rc = N.lib().fp_hybrid_row_limits(ids.data_ptr(), ids.shape[0], soi_id, eoi_id, out.data_ptr(),
+                                      N.stream_ptr(ids.device))
+    N.check(rc, "fp_hybrid_row_limits")
+    return out
+
+
+def paged_prefill(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor, batch_idx: Tensor,
+                  input_pos: Tensor, row_limit: Tensor, page_size: int, *, scale: float | None = None,
+                  out: Tensor | None = None, lse: Tensor | None = None) -> tuple[Tensor, Tensor]:
+    """Chunked-prefill attention over the paged cache.  q [1, Hq, Lq, D]; returns out like q, lse [1, Hq, Lq]."""
+    N.require_cuda(q, pool_k, pool_v, page_table, batch_idx, input_pos, row_limit, out, lse)
+    one, Hq, Lq, D = q.shape
+    if one != 1:
+        raise RuntimeError("paged_prefill takes the packed layout [1, Hq, Lq, D]")
+    Hc, n_slots, Dp = pool_k.shape
+    if Dp != D or pool_k.dtype != q.dtype or pool_v.dtype != q.dtype:
+        raise RuntimeError("q / pool shape or dtype mismatch")
+    q = _rows(q)
+    batch_idx = batch_idx.reshape(-1).contiguous()
+    input_pos = input_pos.reshape(-1).contiguous()
+    row_limit = row_limit.reshape(-1).contiguous()
+    if batch_idx.dtype != torch.int64 or input_pos.dtype != torch.int64 or row_limit.dtype != torch.int32:
+        raise RuntimeError("batch_idx, input_pos must be int64 and row_limit int32")
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    if out is None:
+        out = torch.empty_like(q)
+    if lse is None:
+        lse = torch.empty((1, Hq, Lq), dtype=torch.float32, device=q.device)
+    if out.stride(3) != 1 or not lse.is_contiguous():
+        raise RuntimeError("out rows must be dense and lse contiguous")
+    rc = N.lib().fp_paged_prefill(
+        q.data_ptr(), q.stride(2), q.stride(1), pool_k.data_ptr(), pool_v.data_ptr(),
+        page_table.data_ptr(), page_table.stride(0), batch_idx.data_ptr(), input_pos.data_ptr(),
+        row_limit.data_ptr(), out.data_ptr(), out.stride(2), out.stride(1), lse.data_ptr(),
+        Lq, Hq, Hc, D, page_size, page_table.shape[1], page_table.shape[0], n_slots,
+        scale, N.dtype_code(q.dtype), N.stream_ptr(q.device))
+    N.check(rc, "fp_paged_prefill")
+    return out, lse

@@ -1,0 +1,211 @@
+/*
+ * fp_paged_kv.h -- C ABI of libfp_paged_kv.so: the paged KV-cache path of
+ * Falcon Perception as hand-written HIP kernels for gfx950 (MI355X).
+ *
+ * The reference implements this path in Python on top of torch
+ * (falcon_perception/paged_attention.py, falcon_perception/attention.py); it has
+ * no FFI of its own, so each entry point below names the reference function
+ * whose device work it replaces.
+ *
+ * Conventions
+ *  - Every pointer is a DEVICE pointer owned by the caller.  The library
+ *    borrows it for the duration of the launch; it allocates and frees nothing.
+ *  - `stream` is a hipStream_t passed as void*.  All work is enqueued on it,
+ *    nothing synchronises, so every entry point may be captured in a HIP graph.
+ *  - Strides are in ELEMENTS of the tensor's dtype, the innermost (head_dim)
+ *    stride must be 1.
+ *  - Return value: 0 on success, a negative FP_ERR_* code otherwise;
+ *    fp_last_error() then holds a message for the calling thread.
+ *  - Indices that fall outside the tables or the pool (a slot < 0 or >= n_slots,
+ *    a batch index >= max_batch, a block id >= n_pages) are skipped on the
+ *    device instead of faulting; the reference raises an index error there.
+ */
+#ifndef FP_PAGED_KV_H
+#define FP_PAGED_KV_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FP_ABI_VERSION 1
+
+/* element types of pool / q / k / v */
+#define FP_DTYPE_F32 0
+#define FP_DTYPE_BF16 1
+#define FP_DTYPE_F16 2
+
+/* integer width of position / length arrays */
+#define FP_INDEX_I32 0
+#define FP_INDEX_I64 1
+
+#define FP_OK 0
+#define FP_ERR_INVALID_ARGUMENT (-1)
+#define FP_ERR_UNSUPPORTED (-2)
+#define FP_ERR_LAUNCH (-3)
+#define FP_ERR_WORKSPACE (-4)
+
+/* ABI version of the loaded library (FP_ABI_VERSION at build time). */
+int fp_abi_version(void);
+
+/* Message of the last failing call on this thread ("" if none). */
+const char* fp_last_error(void);
+
+/*
+ * KV append: slot-mapping scatter of new K/V rows into the page pool.
+ * Replaces PagedKVCache.assign (paged_attention.py:184-232; clamp_negative = 1:
+ * stale -1 table entries go to page 0, :222) and
+ * PagedKVCache.assign_prefill_no_paging (paged_attention.py:364-393;
+ * clamp_negative = 0: a negative slot wraps from the end of the slot axis as the
+ * reference's negative index does, :389-391).
+ *
+ *   pool_k, pool_v   [H, n_slots, D]   one layer's K and V planes of kv_cache
+ *   k, v             [T, H, S, D] with element strides (t, h, s); bytes are copied
+ *                    unchanged.  Prefill [1, H, L, D] is passed as T = L, S = 1,
+ *                    stride_t = the stride of the L axis.
+ *   page_table       [max_batch, n_pages] int64, row stride pt_row_stride
+ *   batch_idx        [T] int64  cache slot of each row group
+ *   input_pos        [T, S] contiguous, int32 or int64 (pos_index_type)
+ * Row (t, s) of head h goes to
+ *   pool[h, page_table[batch_idx[t], pos / page_size] * page_size + pos % page_size, :].
+ */
+int fp_kv_append(void* pool_k, void* pool_v,
+                 const void* k, const void* v,
+                 int64_t k_stride_t, int64_t k_stride_h, int64_t k_stride_s,
+                 int64_t v_stride_t, int64_t v_stride_h, int64_t v_stride_s,
+                 const int64_t* page_table, int64_t pt_row_stride,
+                 const int64_t* batch_idx,
+                 const void* input_pos, int pos_index_type,
+                 int32_t T, int32_t H, int32_t S, int32_t D,
+                 int32_t page_size, int32_t n_pages, int32_t max_batch,
+                 int64_t n_slots, int dtype, int clamp_negative,
+                 void* stream);
+
+/*
+ * Page gather: the logical view of cached sequences, the inverse of fp_kv_append.
+ * The reference gathers pages implicitly inside its attention kernels through the
+ * converted block indices (paged_attention.py:279-284); this is that lookup as a
+ * standalone bit copy.
+ *
+ *   pool   [H, n_slots, D]
+ *   out    [B, H, max_len, D] with element strides (b, h, t)
+ *   out[b, h, t, :] = pool[h, page_table[batch_idx[b], t / P] * P + t % P, :]
+ *                     for t < seq_lens[b], zero for seq_lens[b] <= t < max_len.
+ */
+int fp_kv_gather(const void* pool, void* out,
+                 int64_t out_stride_b, int64_t out_stride_h, int64_t out_stride_t,
+                 const int64_t* page_table, int64_t pt_row_stride,
+                 const int64_t* batch_idx,
+                 const void* seq_lens, int len_index_type,
+                 int32_t B, int32_t H, int32_t max_len, int32_t D,
+                 int32_t page_size, int32_t n_pages, int32_t max_batch,
+                 int64_t n_slots, int dtype,
+                 void* stream);
+
+/*
+ * Logical -> physical block ids of a block mask.
+ * Replaces the zeros + torch.gather pair in
+ * PagedKVCache.convert_logical_block_mask (paged_attention.py:279-284).
+ *
+ *   kv_indices   [B, rows_per_batch, C] int32 contiguous (rows_per_batch = H*ROWS)
+ *   out          [B, rows_per_batch, n_pages] int32 contiguous
+ *   out[b, r, c] = (int32) page_table[batch_idx[b], kv_indices[b, r, c]] for c < C, else 0.
+ */
+int fp_convert_block_ids(const int32_t* kv_indices, int32_t* out,
+                         const int64_t* page_table, int64_t pt_row_stride,
+                         const int64_t* batch_idx,
+                         int32_t B, int32_t rows_per_batch, int32_t C,
+                         int32_t n_pages, int32_t max_batch,
+                         void* stream);
+
+/*
+ * Split size (tokens per split-K partition) fp_paged_decode picks when called with
+ * split_tokens = 0 for this shape; use it to size the workspace.
+ */
+int32_t fp_paged_decode_default_split(int32_t B, int32_t Hc, int32_t max_context, int32_t page_size);
+
+/*
+ * Bytes of workspace fp_paged_decode needs for the given launch shape
+ * (split-K partial results: B * Hq * ceil(max_context / split_tokens) * (D + 2) floats;
+ * nothing when one split covers max_context).  max_context bounds input_pos + 1,
+ * split_tokens is an explicit multiple of 64.
+ * Returns a negative FP_ERR_* code for a bad argument.
+ */
+int64_t fp_paged_decode_workspace_bytes(int32_t B, int32_t Hq, int32_t D,
+                                        int32_t max_context, int32_t split_tokens);
+
+/*
+ * Split-K paged decode attention (one query token per sequence) + cross-split merge.
+ * Replaces compiled_flex_attn_decode (attention.py:17) as called at
+ * model.py:156-162 on the pool views returned by PagedKVCache.assign, together
+ * with the per-step mask plumbing it depends on (paged_inference.py:783-826,
+ * paged_attention.py:234-333): pages are looked up in page_table directly.
+ *
+ *   q        [B, Hq, 1, D], element strides (b, h)
+ *   pool_k/v [Hc, n_slots, D], Hq % Hc == 0; query head h reads cache head h / (Hq/Hc)
+ *   input_pos[B] int32/int64: sequence b attends logical positions 0..input_pos[b]
+ *   out      [B, Hq, 1, D] same dtype as q, element strides (b, h)
+ *   lse      [B, Hq] float32, natural log of the softmax denominator
+ *   scale    multiplies q.k (1/sqrt(D) in the reference)
+ *   max_context   upper bound of input_pos + 1, fixes the launch grid
+ *   split_tokens  tokens per split, a multiple of 64 (0 = library default)
+ * A sequence with input_pos < 0 yields out = 0, lse = -inf.
+ */
+int fp_paged_decode(const void* q, int64_t q_stride_b, int64_t q_stride_h,
+                    const void* pool_k, const void* pool_v,
+                    const int64_t* page_table, int64_t pt_row_stride,
+                    const int64_t* batch_idx,
+                    const void* input_pos, int pos_index_type,
+                    void* out, int64_t out_stride_b, int64_t out_stride_h,
+                    float* lse,
+                    void* workspace, int64_t workspace_bytes,
+                    int32_t B, int32_t Hq, int32_t Hc, int32_t D,
+                    int32_t page_size, int32_t n_pages, int32_t max_batch,
+                    int64_t n_slots, int32_t max_context, int32_t split_tokens,
+                    float scale, int dtype,
+                    void* stream);
+
+/*
+ * Per-row key limits of the hybrid mask (bidirectional inside an image span,
+ * causal elsewhere).  Replaces the compiled create_block_mask evaluation of
+ * create_prefill_blockmask (paged_attention.py:343-362) with
+ * get_image_prefix_mask_mod (attention.py:75-96) by a closed form.
+ *
+ *   input_ids [L] int64 packed token ids, soi_id / eoi_id the span delimiters
+ *   row_hi    [L] int32 out: packed index one past the last key row q may see
+ *             = max(q + 1, end of q's image span)
+ * L <= 65536 (one workgroup scans the row).
+ */
+int fp_hybrid_row_limits(const int64_t* input_ids, int32_t L,
+                         int64_t soi_id, int64_t eoi_id,
+                         int32_t* row_hi, void* stream);
+
+/*
+ * Chunked-prefill attention over the paged cache under the hybrid mask (bf16/f16 MFMA).
+ * Replaces compiled_flex_attn_prefill (attention.py:18) as called at model.py:156-162,
+ * extended to read the prefix from pages (the reference attends over the packed
+ * fresh K/V only, paged_attention.py:393).
+ *
+ *   q          [Lq, Hq, D] view with element strides (row, head) of the packed rows
+ *   batch_idx  [Lq] int64 cache slot of each row (0 = padding: out 0, lse -inf)
+ *   input_pos  [Lq] int64 logical position of each row in its sequence
+ *   row_limit  [Lq] int32 logical keys 0..row_limit-1 of the row's sequence are visible
+ *   out        [Lq, Hq, D] view, strides (row, head); lse [Hq, Lq] float32
+ */
+int fp_paged_prefill(const void* q, int64_t q_stride_row, int64_t q_stride_h,
+                     const void* pool_k, const void* pool_v,
+                     const int64_t* page_table, int64_t pt_row_stride,
+                     const int64_t* batch_idx, const int64_t* input_pos,
+                     const int32_t* row_limit,
+                     void* out, int64_t out_stride_row, int64_t out_stride_h,
+                     float* lse,
+                     int32_t Lq, int32_t Hq, int32_t Hc, int32_t D,
+                     int32_t page_size, int32_t n_pages, int32_t max_batch,
+                     int64_t n_slots, float scale, int dtype,
+                     void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FP_PAGED_KV_H */

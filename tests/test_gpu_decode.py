@@ -1,0 +1,201 @@
+"""GPU parity: split-K paged decode attention against the float64 oracle.
+
+Tolerance (north star): 2e-2 absolute / 1e-2 relative for bf16; fp32 and fp16 are
+held to tighter bounds written next to each check.
+"""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+from torch.nn.attention.flex_attention import AuxRequest, BlockMask
+
+from falcon_perception_amd import attention as A
+from falcon_perception_amd import ops
+from oracle import paged_kv_oracle as O
+from tests.gpu_cases import DEV, PagedState, f64, randn
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.bfloat16: (2e-2, 1e-2), torch.float16: (2e-3, 2e-3), torch.float32: (2e-5, 2e-5)}
+
+
+def run_decode(st, q, pos, **kw):
+    pk, pv = st.pool_planes()
+    bidx = torch.tensor(st.slots, dtype=torch.int64, device=DEV)
+    max_ctx = kw.pop("max_context", st.cache.n_pages * st.P)
+    return ops.paged_decode(q.to(DEV), pk, pv, st.cache.page_table, bidx, pos.to(DEV), st.P, max_ctx, **kw)
+
+
+def oracle_decode(st, q, pos):
+    pk, pv = st.pool_planes()
+    return O.decode_attention(f64(q), f64(pk), f64(pv), st.mirror.page_table, st.slots, pos.numpy(), st.P)
+
+
+def assert_close(out, lse, eo, el, dtype):
+    atol, rtol = TOL[dtype]
+    np.testing.assert_allclose(f64(out), eo, atol=atol, rtol=rtol)
+    np.testing.assert_allclose(f64(lse), el, atol=max(atol * 0.1, 1e-5), rtol=rtol)
+
+
+def test_cfg1_cpu_reference_shape_fp32():
+    """BASELINE configs[0]: 64 pages x 64, 8 heads x 64, fp32, batch 4, contexts U[64,512],
+    append one token per sequence then decode."""
+    st = PagedState(1, n_pages=64, page_size=64, max_batch=8, Hc=8, D=64, dtype=torch.float32)
+    lens = torch.randint(64, 513, (4,), generator=st.gen).tolist()
+    for L in lens:
+        st.add_sequence(L + 1)  # room for the appended token
+    st.lens = lens
+    st.prefill_random()
+    k = randn(st.gen, (4, 8, 1, 64), torch.float32)
+    v = randn(st.gen, (4, 8, 1, 64), torch.float32)
+    q = randn(st.gen, (4, 8, 1, 64), torch.float32)
+    pos = torch.tensor(lens, dtype=torch.int32)  # the new token's position
+    bidx = torch.tensor(st.slots, dtype=torch.int64, device=DEV)
+    st.cache.insert_kv(0, k.to(DEV), v.to(DEV), input_pos=pos.view(4, 1).to(DEV), batch_idx=bidx)
+    out, lse = run_decode(st, q, pos)
+    eo, el = oracle_decode(st, q, pos)
+    assert_close(out, lse, eo, el, torch.float32)
+    assert out.dtype == torch.float32 and lse.dtype == torch.float32 and lse.shape == (4, 8, 1)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=str)
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("G", [1, 2, 4, 8])
+def test_context_boundaries_and_gqa(dtype, D, G):
+    P = 16
+    st = PagedState(2, n_pages=80, page_size=P, max_batch=12, Hc=2, D=D, dtype=dtype)
+    lens = [1, 2, P - 1, P, P + 1, 4 * P, 4 * P + 1, 63, 64, 65, 300]
+    for L in lens:
+        st.add_sequence(L)
+    st.prefill_random()
+    q = randn(st.gen, (len(lens), 2 * G, 1, D), dtype)
+    pos = torch.tensor([L - 1 for L in lens], dtype=torch.int32)
+    eo, el = oracle_decode(st, q, pos)
+    for split in (0, 64, 128):
+        out, lse = run_decode(st, q, pos, split_tokens=split, max_context=320)
+        assert_close(out, lse, eo, el, dtype)
+
+
+def test_no_visible_key_and_int64_positions():
+    dtype = torch.bfloat16
+    st = PagedState(3, n_pages=32, page_size=16, max_batch=6, Hc=2, D=128, dtype=dtype)
+    for L in (40, 70, 9):
+        st.add_sequence(L)
+    st.prefill_random()
+    q = randn(st.gen, (3, 4, 1, 128), dtype)
+    pos = torch.tensor([39, -1, 8], dtype=torch.int64)
+    for ctx in (64, 512):  # single-split (direct) and split-K + merge paths
+        out, lse = run_decode(st, q, pos, max_context=ctx)
+        eo, el = oracle_decode(st, q, pos)
+        assert_close(out[[0, 2]], lse[[0, 2]], eo[[0, 2]], el[[0, 2]], dtype)
+        assert not out[1].any() and torch.isneginf(lse[1]).all()
+
+
+def test_page_permutation_and_split_invariance():
+    """Same logical content under two page tables gives identical results bit for bit;
+    different split sizes agree to fp32 rounding."""
+    dtype = torch.bfloat16
+    outs = []
+    for shuffle in (False, True):
+        st = PagedState(4, n_pages=64, page_size=32, max_batch=6, Hc=4, D=128, dtype=dtype, shuffle=shuffle)
+        gen = torch.Generator().manual_seed(44)
+        st.gen = gen  # identical K/V/q for both layouts
+        for L in (500, 37, 960):
+            st.add_sequence(L)
+        st.prefill_random()
+        q = randn(gen, (3, 8, 1, 128), dtype)
+        pos = torch.tensor([499, 36, 959], dtype=torch.int32)
+        outs.append(run_decode(st, q, pos, split_tokens=256, max_context=1024))
+        if shuffle:
+            o64 = run_decode(st, q, pos, split_tokens=64, max_context=1024)
+            o1k = run_decode(st, q, pos, split_tokens=1024, max_context=1024)
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+    np.testing.assert_allclose(f64(o64[1]), f64(o1k[1]), atol=1e-5, rtol=1e-5)
+    np.testing.assert_allclose(f64(o64[0]), f64(o1k[0]), atol=8e-3, rtol=8e-3)  # one bf16 ulp of the output
+
+
+def test_strided_query_and_preallocated_outputs():
+    dtype = torch.bfloat16
+    st = PagedState(5, n_pages=32, page_size=16, max_batch=4, Hc=2, D=128, dtype=dtype)
+    st.add_sequence(130)
+    st.add_sequence(77)
+    st.prefill_random()
+    # q as the model produces it: [B, S, H, D] memory viewed as [B, H, S, D]
+    q = randn(st.gen, (2, 1, 4, 128), dtype).to(DEV).permute(0, 2, 1, 3)
+    assert not q.is_contiguous() or q.shape[2] == 1
+    pos = torch.tensor([129, 76], dtype=torch.int32)
+    out = torch.zeros((2, 1, 4, 128), dtype=dtype, device=DEV).permute(0, 2, 1, 3)
+    lse = torch.zeros((2, 4, 1), dtype=torch.float32, device=DEV)
+    r_out, r_lse = run_decode(st, q, pos, out=out, lse=lse, max_context=256)
+    assert r_out.data_ptr() == out.data_ptr()
+    eo, el = oracle_decode(st, q.cpu(), pos)
+    assert_close(out, lse, eo, el, dtype)
+
+
+def test_cfg2_serving_shape_bf16():
+    """BASELINE configs[1] at full size: batch 64, 16 q / 8 kv heads, D 128, page 128,
+    contexts 1024 + U[64,3072], fragmented 4096-page pool."""
+    import bench
+
+    case = bench.make_decode_case("cfg2", device=DEV)
+    out, lse = case.run()
+    f32 = lambda t: t.float().cpu().numpy()  # exact for bf16; the oracle widens per sequence
+    eo, el = O.decode_attention(f64(case.q), f32(case.pool_k), f32(case.pool_v), case.page_table.cpu().numpy(),
+                                case.batch_idx.cpu().numpy(), case.input_pos.cpu().numpy(), case.page_size)
+    assert_close(out, lse, eo, el, torch.bfloat16)
+
+
+def test_attention_callable_with_engine_masks():
+    """The reference's call: insert_kv then compiled_flex_attn_decode(q, K, V, block_mask, return_aux)
+    (model.py:150-162) with the mask built as paged_inference.py:783-848 builds it."""
+    dtype = torch.bfloat16
+    P, Lmax, H, D = 16, 256, 4, 128
+    st = PagedState(6, n_pages=64, page_size=P, max_batch=8, Hc=H, D=D, dtype=dtype)
+    lens = [100, 17, 255, 33]
+    for L in lens:
+        st.add_sequence(L + 1)
+    st.lens = lens
+    st.prefill_random()
+    cache = st.cache
+    full = cache.create_causal_blockmask(B=8, L=Lmax)
+    # two padded rows with batch slot 0 as CUDA-graph buckets have (paged_inference.py:970-992)
+    bidx = torch.tensor(st.slots + [0, 0], dtype=torch.int64, device=DEV)
+    input_pos_all = torch.zeros(8, dtype=torch.int32, device=DEV)
+    input_pos_all[torch.tensor(st.slots, device=DEV)] = torch.tensor(lens, dtype=torch.int32, device=DEV)
+    pos = input_pos_all[bidx]
+    B = 6
+    blk = pos // P
+    step = BlockMask.from_kv_blocks(
+        full.kv_num_blocks[bidx, :, blk].view(B, 1, 1), full.kv_indices[bidx, :, blk].view(B, 1, 1, -1),
+        full.full_kv_num_blocks[bidx, :, blk].view(B, 1, 1), full.full_kv_indices[bidx, :, blk].view(B, 1, 1, -1),
+        BLOCK_SIZE=full.BLOCK_SIZE, mask_mod=lambda b, h, q, kv: q + pos[b] >= kv, seq_lengths=(1, Lmax))
+    mask = cache.convert_logical_block_mask(step, bidx)
+    k = randn(st.gen, (B, H, 1, D), dtype).to(DEV)
+    v = randn(st.gen, (B, H, 1, D), dtype).to(DEV)
+    q = randn(st.gen, (B, H, 1, D), dtype).to(DEV)
+    K, V = cache.insert_kv(0, k, v, input_pos=pos.view(B, 1), batch_idx=bidx)
+    out, aux = A.compiled_flex_attn_decode(q, K, V, block_mask=mask, return_aux=AuxRequest(lse=True),
+                                           kernel_options={"BLOCK_M": 64, "BLOCK_N": 64, "num_stages": 1})
+    assert out.shape == (B, H, 1, D) and aux.lse.shape == (B, H, 1)
+    eo, el = O.decode_attention(f64(q[:4]), f64(K[0]), f64(V[0]), cache.page_table.cpu().numpy(),
+                                st.slots, np.array(lens), P)
+    assert_close(out[:4], aux.lse[:4], eo, el, dtype)
+    assert torch.isfinite(out.float()).all()  # padded rows read page 0 and stay finite
+    # the same step through a captured HIP graph, replayed with new positions
+    g = torch.cuda.CUDAGraph()
+    static_q = q.clone()
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        A.compiled_flex_attn_decode(static_q, K, V, block_mask=mask, return_aux=AuxRequest(lse=True))
+    torch.cuda.current_stream().wait_stream(s)
+    with torch.cuda.graph(g):
+        g_out, g_aux = A.compiled_flex_attn_decode(static_q, K, V, block_mask=mask, return_aux=AuxRequest(lse=True))
+    for trial in range(3):
+        static_q.copy_(randn(st.gen, (B, H, 1, D), dtype))
+        g.replay()
+        torch.cuda.synchronize()
+        e_out, e_aux = A.compiled_flex_attn_decode(static_q, K, V, block_mask=mask, return_aux=AuxRequest(lse=True))
+        assert torch.equal(g_out, e_out) and torch.equal(g_aux.lse, e_aux.lse)

@@ -1,0 +1,216 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports what the
+header declares, the Python mirror keeps the reference's allocator semantics and
+mask structure, and nothing silently falls back to a CPU path."""
+
+import json
+import os
+import random
+import re
+import sys
+
+import numpy as np
+import pytest
+import torch
+from torch.nn.attention.flex_attention import create_block_mask
+
+import falcon_perception_amd as fpa
+from falcon_perception_amd import _native
+from falcon_perception_amd import attention as A
+from falcon_perception_amd.paged_attention import PagedKVCache
+from oracle import paged_kv_oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def header_functions():
+    text = open(os.path.join(ROOT, "include", "fp_paged_kv.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fp_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(native_lib):
+    names = header_functions()
+    assert len(names) >= 9
+    for n in names:
+        assert hasattr(native_lib, n), f"{n} declared in the header but not exported"
+    assert sorted(_native.SIGNATURES) == names
+    assert native_lib.fp_abi_version() == _native.FP_ABI_VERSION
+
+
+def test_argument_errors_come_back_as_codes_not_crashes(native_lib):
+    # no device work: every call below is rejected by the host-side checks
+    assert native_lib.fp_paged_decode_workspace_bytes(4, 8, 128, 1024, 100) < 0  # split not a multiple of 64
+    assert b"multiple of 64" in native_lib.fp_last_error()
+    assert native_lib.fp_paged_decode_workspace_bytes(4, 8, 128, 1024, 256) == 4 * 8 * 4 * 130 * 4
+    assert native_lib.fp_paged_decode_workspace_bytes(4, 8, 128, 256, 256) == 0  # one split: no workspace
+    assert native_lib.fp_paged_decode_default_split(64, 8, 4096, 128) % 64 == 0
+    rc = native_lib.fp_kv_append(None, None, None, None, 0, 0, 0, 0, 0, 0, None, 0, None, None, 0,
+                                 4, 2, 1, 8, 4, 8, 4, 32, 7, 1, None)
+    assert rc == -2 and b"dtype" in native_lib.fp_last_error()
+    rc = native_lib.fp_kv_append(None, None, None, None, 0, 0, 0, 0, 0, 0, None, 0, None, None, 0,
+                                 4, 2, 1, 8, 4, 8, 4, 32, 1, 1, None)
+    assert rc == -1 and b"null" in native_lib.fp_last_error()
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(_native, "_lib", None)
+    monkeypatch.setattr(_native, "LIB_PATH", "/nonexistent/libfp_paged_kv.so")
+    with pytest.raises(RuntimeError, match="no other compute path"):
+        _native.lib()
+
+
+def test_no_cpu_fallback():
+    c = PagedKVCache(8, 4, 4, 2, 8, 1, torch.float32, device="cpu")
+    b = c.allocate()
+    c.reserve(b, torch.tensor([b]), 4)
+    k = torch.zeros(1, 2, 1, 8)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        c.insert_kv(0, k, k, input_pos=torch.zeros(1, 1, dtype=torch.int32), batch_idx=torch.tensor([b]))
+
+
+def snapshot(c):
+    return (list(c.free_pages), list(c.free_batch_idx), list(c.capacity),
+            [list(x) for x in c.page_table_cpu], c.page_table.tolist(), c.physical_to_logical.tolist())
+
+
+def o_snapshot(a):
+    return (list(a.free_pages), list(a.free_batch_idx), list(a.capacity),
+            [list(x) for x in a.page_table_cpu], a.page_table.tolist(), a.physical_to_logical.tolist())
+
+
+def test_allocator_known_answers():
+    cases = json.load(open(os.path.join(ROOT, "tests", "golden", "allocator_kat.json")))["cases"]
+    for case in cases:
+        i = case["init"]
+        c = PagedKVCache(i["n_pages"], i["page_size"], i["max_batch_size"], 1, 4, 1, torch.float32, device="cpu")
+        got = []
+        for op in case["trace"]:
+            if op[0] == "allocate":
+                got.append(c.allocate())
+            elif op[0] == "reserve":
+                got.append(c.reserve(op[1], torch.tensor([op[1]]), op[2]))
+            elif op[0] == "erase":
+                c.erase(op[1])
+                got.append(None)
+            else:
+                got.append(c.can_reserve(op[1], op[2] if len(op) > 2 else None))
+        assert got == case["returns"], case["name"]
+        f = case["final"]
+        assert snapshot(c) == (f["free_pages"], f["free_batch_idx"], f["capacity"], f["page_table_cpu"],
+                               f["page_table"], f["physical_to_logical"]), case["name"]
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_allocator_follows_the_oracle_on_random_traces(seed):
+    rng = random.Random(seed)
+    c = PagedKVCache(33, 8, 9, 1, 4, 1, torch.float32, device="cpu")
+    a = O.PagedAllocator(33, 8, 9)
+    assert c.kv_cache.shape == (1, 2, 1, 1, 33 * 8, 4) and c.kv_shape == tuple(c.kv_cache.shape)
+    live, want = [], {}
+    for _ in range(300):
+        r = rng.random()
+        if r < 0.25 and c.free_batch_idx and c.can_reserve(1):
+            b = c.allocate()
+            assert b == a.allocate()
+            live.append(b)
+            want[b] = 0
+        elif r < 0.75 and live:
+            b = rng.choice(live)
+            n = want[b] + rng.randint(1, 20)
+            assert c.can_reserve(n, b) == a.can_reserve(n, b)
+            if c.can_reserve(n, b):
+                c.reserve(b, torch.tensor([b]), n)
+                a.reserve(b, n)
+                want[b] = n
+            else:
+                with pytest.raises(RuntimeError) as e1:
+                    c.reserve(b, torch.tensor([b]), n)
+                with pytest.raises(RuntimeError) as e2:
+                    a.reserve(b, n)
+                assert str(e1.value) == str(e2.value)
+        elif live:
+            b = live.pop(rng.randrange(len(live)))
+            c.erase(b)
+            a.erase(b)
+            del want[b]
+        assert snapshot(c) == o_snapshot(a)
+        assert c.num_free_pages == a.num_free_pages
+
+
+@pytest.mark.parametrize("n_blocks", [1, 3, 8])
+def test_causal_blockmask_equals_torch_create_block_mask(n_blocks):
+    P, B = 4, 3
+    c = PagedKVCache(16, P, 4, 1, 4, 1, torch.float32, device="cpu")
+    L = n_blocks * P
+    got = c.create_causal_blockmask(B, L)
+    ref = create_block_mask(A.get_causal_mask_mod(), B, None, L, L, device="cpu", BLOCK_SIZE=P)
+    assert got.BLOCK_SIZE == ref.BLOCK_SIZE and got.seq_lengths == ref.seq_lengths
+    assert got.kv_indices.shape == ref.kv_indices.shape and got.kv_indices.dtype == ref.kv_indices.dtype
+    assert torch.equal(got.kv_num_blocks, ref.kv_num_blocks)
+    assert torch.equal(got.kv_indices, ref.kv_indices)
+    if n_blocks > 1:
+        assert torch.equal(got.full_kv_num_blocks, ref.full_kv_num_blocks)
+        assert torch.equal(got.full_kv_indices, ref.full_kv_indices)
+    assert torch.equal(got.to_dense(), ref.to_dense())
+    # the engine slices it like this (reference paged_inference.py:803-826)
+    bidx = torch.tensor([2, 1])
+    blk = torch.tensor([0, n_blocks - 1])
+    assert got.kv_num_blocks[bidx, :, blk].shape == (2, 1)
+    assert got.kv_indices[bidx, :, blk].view(2, 1, 1, -1).shape == (2, 1, 1, n_blocks)
+
+
+def test_convert_rejects_a_foreign_block_size():
+    c = PagedKVCache(16, 4, 4, 1, 4, 1, torch.float32, device="cpu")
+    other = PagedKVCache(16, 8, 4, 1, 4, 1, torch.float32, device="cpu").create_causal_blockmask(2, 16)
+    with pytest.raises(RuntimeError, match="same column block size"):
+        c.convert_logical_block_mask(other)
+
+
+def test_physical_mask_mod_matches_the_oracle():
+    c = PagedKVCache(10, 4, 4, 1, 4, 1, torch.float32, device="cpu")
+    c.free_pages = [3, 8, 1, 6, 9, 2, 7, 5, 4]
+    slots = []
+    for L in (6, 9):
+        b = c.allocate()
+        c.reserve(b, torch.tensor([b]), L)
+        slots.append(b)
+    bidx = torch.tensor(slots)
+    mod = c.get_mask_mod(A.get_causal_mask_mod(), bidx)
+    p2l = c.physical_to_logical.numpy()
+    for b in range(2):
+        for q in (0, 5):
+            phys = torch.arange(40)
+            got = mod(torch.tensor(b), torch.tensor(0), torch.tensor(q), phys)
+            exp = [O.physical_mask(p2l, slots, 4, lambda _b, qq, kv: qq >= kv, b, q, int(p)) for p in phys]
+            assert got.tolist() == exp
+
+
+def test_mask_mod_factories_match_the_oracle_tables():
+    from tests.test_oracle_masks import EOI, SOI, packed_case
+
+    ids, bidx, pos, spans = packed_case([(1, [("t", 2), ("i", 5), ("t", 3)]), (2, [("i", 3), ("t", 2)])])
+    t_ids = torch.from_numpy(ids)[None]
+    mod = A.get_image_prefix_mask_mod(t_ids, SOI, EOI)
+    L = len(ids)
+    qq, kk = torch.meshgrid(torch.arange(L), torch.arange(L), indexing="ij")
+    got = mod(torch.tensor(0), torch.tensor(0), qq, kk).numpy()
+    img, idx = O.image_prefix_tables(ids, SOI, EOI)
+    exp = img[:, None] & img[None, :] & (idx[:, None] == idx[None, :])
+    assert np.array_equal(got, exp)
+    assert A.offset_mask_mod(A.get_causal_mask_mod(), 3)(0, 0, torch.tensor(1), torch.tensor(4)).item()
+
+
+def test_install_serves_the_reference_module_names():
+    saved = {k: sys.modules.get(k) for k in
+             ("falcon_perception.kv_cache", "falcon_perception.paged_attention", "falcon_perception.attention")}
+    try:
+        fpa.install()
+        assert sys.modules["falcon_perception.paged_attention"].PagedKVCache is PagedKVCache
+        assert sys.modules["falcon_perception.attention"].compiled_flex_attn_decode is A.compiled_flex_attn_decode
+        assert sys.modules["falcon_perception.kv_cache"].KVCacheBase is fpa.KVCacheBase
+    finally:
+        for k, v in saved.items():
+            if v is None:
+                sys.modules.pop(k, None)
+            else:
+                sys.modules[k] = v
