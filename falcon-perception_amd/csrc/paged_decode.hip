@@ -57,11 +57,27 @@ struct DecodeArgs {
   float qscale;  // scale * log2(e)
 };
 
-// ---- element access: 16 bytes of a row as floats -------------------------
+// ---- element access: 16 bytes of a row -----------------------------------
+// A lane holds 16 bytes of a K or V row as four 32-bit words.  `Q` is the lane's
+// share of a query row, `dot` its contribution to q.k, `unpack` the V values as floats.
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+
 struct F32 {
   using type = float;
   static constexpr int kEpl = 4;
-  static __device__ __forceinline__ void unpack(const uint4& r, float* f) {
+  struct Q { float f[4]; };
+  static __device__ __forceinline__ Q load_q(const v4u& r) {
+    return Q{{__uint_as_float(r.x), __uint_as_float(r.y), __uint_as_float(r.z), __uint_as_float(r.w)}};
+  }
+  static __device__ __forceinline__ float dot(const Q& q, const v4u& k) {
+    float p = q.f[0] * __uint_as_float(k.x);
+    p = fmaf(q.f[1], __uint_as_float(k.y), p);
+    p = fmaf(q.f[2], __uint_as_float(k.z), p);
+    return fmaf(q.f[3], __uint_as_float(k.w), p);
+  }
+  static __device__ __forceinline__ void unpack(const v4u& r, float* f) {
     f[0] = __uint_as_float(r.x);
     f[1] = __uint_as_float(r.y);
     f[2] = __uint_as_float(r.z);
@@ -69,15 +85,27 @@ struct F32 {
   }
   static __device__ __forceinline__ void store(char* p, float v) { *reinterpret_cast<float*>(p) = v; }
 };
+// bf16 / f16: q.k on the packed pairs with v_dot2 (fp32 accumulate), no conversion of K
 struct BF16 {
   using type = __hip_bfloat16;
   static constexpr int kEpl = 8;
-  static __device__ __forceinline__ void unpack(const uint4& r, float* f) {
-    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+  struct Q { v4u w; };
+  static __device__ __forceinline__ Q load_q(const v4u& r) { return Q{r}; }
+  static __device__ __forceinline__ float dot(const Q& q, const v4u& k) {
+    float p = 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      f[2 * i] = __uint_as_float(w[i] << 16);
-      f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+      // the words go through scalars: bit_cast applied directly to a vector element reads element 0
+      const uint32_t qw = q.w[i], kw = k[i];
+      p = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, qw), __builtin_bit_cast(bf16x2_t, kw), p, false);
+    }
+    return p;
+  }
+  static __device__ __forceinline__ void unpack(const v4u& r, float* f) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = __uint_as_float(r[i] << 16);
+      f[2 * i + 1] = __uint_as_float(r[i] & 0xffff0000u);
     }
   }
   static __device__ __forceinline__ void store(char* p, float v) {
@@ -87,18 +115,33 @@ struct BF16 {
 struct F16 {
   using type = __half;
   static constexpr int kEpl = 8;
-  static __device__ __forceinline__ void unpack(const uint4& r, float* f) {
-    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+  struct Q { v4u w; };
+  static __device__ __forceinline__ Q load_q(const v4u& r) { return Q{r}; }
+  static __device__ __forceinline__ float dot(const Q& q, const v4u& k) {
+    float p = 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const __half2 h = *reinterpret_cast<const __half2*>(&w[i]);
-      const float2 x = __half22float2(h);
-      f[2 * i] = x.x;
-      f[2 * i + 1] = x.y;
+      const uint32_t qw = q.w[i], kw = k[i];
+      p = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, qw), __builtin_bit_cast(f16x2_t, kw), p, false);
+    }
+    return p;
+  }
+  static __device__ __forceinline__ void unpack(const v4u& r, float* f) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t w = r[i];
+      const f16x2_t h = __builtin_bit_cast(f16x2_t, w);
+      f[2 * i] = static_cast<float>(h.x);
+      f[2 * i + 1] = static_cast<float>(h.y);
     }
   }
   static __device__ __forceinline__ void store(char* p, float v) { *reinterpret_cast<__half*>(p) = __float2half(v); }
 };
+
+// K and V are streamed once: non-temporal loads keep them from displacing the caches
+__device__ __forceinline__ v4u stream_load(const char* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const v4u*>(p));
+}
 
 // ---- cross-lane helpers ---------------------------------------------------
 template <int kCtrl>
@@ -106,23 +149,85 @@ __device__ __forceinline__ float dpp(float x) {
   return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), kCtrl, 0xf, 0xf, true));
 }
 
-// sum over the kLanes consecutive lanes that share a row; every lane gets the total
-template <int kLanes>
-__device__ __forceinline__ float row_sum(float x) {
-  if (kLanes >= 2) x += dpp<0xB1>(x);   // quad_perm [1,0,3,2]
-  if (kLanes >= 4) x += dpp<0x4E>(x);   // quad_perm [2,3,0,1]
-  if (kLanes >= 8) x += dpp<0x141>(x);  // row_half_mirror
-  if (kLanes >= 16) x += dpp<0x140>(x); // row_mirror
-  if (kLanes >= 32) x += __shfl_xor(x, 16);
-  if (kLanes >= 64) x += __shfl_xor(x, 32);
-  return x;
+// Sum over the kLanes consecutive lanes that share a row; every lane gets the total.
+// All kN values advance one butterfly step at a time, so back-to-back DPP
+// instructions are independent of each other.
+template <int kLanes, int kN>
+__device__ __forceinline__ void row_sum(float (&x)[kN]) {
+#pragma unroll
+  for (int i = 0; i < kN; ++i) if (kLanes >= 2) x[i] += dpp<0xB1>(x[i]);   // quad_perm [1,0,3,2]
+#pragma unroll
+  for (int i = 0; i < kN; ++i) if (kLanes >= 4) x[i] += dpp<0x4E>(x[i]);   // quad_perm [2,3,0,1]
+#pragma unroll
+  for (int i = 0; i < kN; ++i) if (kLanes >= 8) x[i] += dpp<0x141>(x[i]);  // row_half_mirror
+#pragma unroll
+  for (int i = 0; i < kN; ++i) if (kLanes >= 16) x[i] += dpp<0x140>(x[i]); // row_mirror
+#pragma unroll
+  for (int i = 0; i < kN; ++i) if (kLanes >= 32) x[i] += __shfl_xor(x[i], 16);
+#pragma unroll
+  for (int i = 0; i < kN; ++i) if (kLanes >= 64) x[i] += __shfl_xor(x[i], 32);
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float safe_max(float m) { return m == -INFINITY ? 0.f : m; }
 
+// One wavefront iteration: U row loads of K and V per lane are already in registers;
+// fold them into the lane group's online-softmax state.  kMasked: rows at or past
+// `t1` (only in the last iteration of a split) get a score of -inf.
+template <typename E, int TPR, int G, int U, int RPW, bool kMasked>
+__device__ __forceinline__ void fold_rows(const v4u (&kreg)[U], const v4u (&vreg)[U], const typename E::Q (&q)[G],
+                                          float qscale, int row0, int t1, float (&m)[G], float (&l)[G],
+                                          float (&acc)[G][E::kEpl]) {
+  constexpr int EPL = E::kEpl;
+  float s[G][U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+#pragma unroll
+    for (int g = 0; g < G; ++g) s[g][u] = E::dot(q[g], kreg[u]);
+  }
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    row_sum<TPR, U>(s[g]);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const float tot = s[g][u] * qscale;
+      s[g][u] = (!kMasked || row0 + u * RPW < t1) ? tot : -INFINITY;
+    }
+  }
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    float mx = m[g];
+#pragma unroll
+    for (int u = 0; u < U; ++u) mx = fmaxf(mx, s[g][u]);
+    const float ms = safe_max(mx);
+    const float alpha = fast_exp2(m[g] - ms);
+    m[g] = mx;
+    float ps = 0.f;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      s[g][u] = fast_exp2(s[g][u] - ms);
+      ps += s[g][u];
+    }
+    l[g] = l[g] * alpha + ps;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) acc[g][e] *= alpha;
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    float vf[EPL];
+    E::unpack(vreg[u], vf);
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) acc[g][e] = fmaf(s[g][u], vf[e], acc[g][e]);
+    }
+  }
+}
+
 // ---- main kernel ------------------------------------------------------------
-template <typename E, int D, int G, bool kDirect>
+// kAligned: the page size is a power of two and a multiple of the rows one
+// wavefront iteration covers, so those rows share one page and one base address.
+template <typename E, int D, int G, bool kDirect, bool kAligned>
 __global__ __launch_bounds__(kThreads) void paged_decode_kernel(const DecodeArgs a) {
   constexpr int EPL = E::kEpl;          // elements per lane
   constexpr int TPR = D / EPL;          // lanes per row
@@ -139,7 +244,7 @@ __global__ __launch_bounds__(kThreads) void paged_decode_kernel(const DecodeArgs
   const int hc = blockIdx.y;
   const int b = blockIdx.z;
   const int tid = threadIdx.x;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
   const int grp = lane / TPR;  // row of this lane inside a wavefront load
   const int col = lane % TPR;  // 16-byte chunk of the row
@@ -178,15 +283,11 @@ __global__ __launch_bounds__(kThreads) void paged_decode_kernel(const DecodeArgs
     }
   }
 
-  // query chunk of every head of the group, pre-scaled into log2 space
-  float qf[G][EPL];
+  // this lane's 16 bytes of the query row of every head of the group
+  typename E::Q q[G];
 #pragma unroll
-  for (int g = 0; g < G; ++g) {
-    const uint4 r = *reinterpret_cast<const uint4*>(a.q + b * a.qs_b + (hc * G + g) * a.qs_h + col * 16);
-    E::unpack(r, qf[g]);
-#pragma unroll
-    for (int e = 0; e < EPL; ++e) qf[g][e] *= a.qscale;
-  }
+  for (int g = 0; g < G; ++g)
+    q[g] = E::load_q(*reinterpret_cast<const v4u*>(a.q + b * a.qs_b + (hc * G + g) * a.qs_h + col * 16));
 
   float m[G], l[G], acc[G][EPL];
 #pragma unroll
@@ -202,72 +303,37 @@ __global__ __launch_bounds__(kThreads) void paged_decode_kernel(const DecodeArgs
 
   __syncthreads();
 
+#pragma nounroll
   for (int c0 = t0 + wave * CH; c0 < t1; c0 += kWaves * CH) {
-    uint4 kreg[U], vreg[U];
-    bool valid[U];
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      int t = c0 + u * RPW + grp;
-      valid[u] = t < t1;
-      if (!valid[u]) t = t1 - 1;
-      int64_t blk;
-      int off;
-      a.pd.split(t, blk, off);
-      const int64_t slot = static_cast<int64_t>(s_pages[blk - blk0]) * a.pd.page_size + off;
-      kreg[u] = *reinterpret_cast<const uint4*>(kbase + slot * ROWB);
-      vreg[u] = *reinterpret_cast<const uint4*>(vbase + slot * ROWB);
-    }
-
-    float s[G][U];
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      float kf[EPL];
-      E::unpack(kreg[u], kf);
-#pragma unroll
-      for (int g = 0; g < G; ++g) {
-        float p = 0.f;
-#pragma unroll
-        for (int e = 0; e < EPL; ++e) p = fmaf(qf[g][e], kf[e], p);
-        s[g][u] = p;
-      }
-    }
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
+    v4u kreg[U], vreg[U];
+    if (kAligned) {
+      // the CH rows of this iteration lie in one page: one base, constant offsets
+      const int page = s_pages[(c0 >> a.pd.shift) - static_cast<int>(blk0)];
+      const int64_t slot = static_cast<int64_t>(page) * a.pd.page_size + (c0 & (a.pd.page_size - 1)) + grp;
+      const char* kp = kbase + slot * ROWB;
+      const char* vp = vbase + slot * ROWB;
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const float tot = row_sum<TPR>(s[g][u]);
-        s[g][u] = valid[u] ? tot : -INFINITY;
+        kreg[u] = stream_load(kp + u * RPW * ROWB);
+        vreg[u] = stream_load(vp + u * RPW * ROWB);
       }
-    }
-
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-      float mx = m[g];
-#pragma unroll
-      for (int u = 0; u < U; ++u) mx = fmaxf(mx, s[g][u]);
-      const float ms = safe_max(mx);
-      const float alpha = fast_exp2(m[g] - ms);
-      m[g] = mx;
-      float ps = 0.f;
+    } else {
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        s[g][u] = fast_exp2(s[g][u] - ms);
-        ps += s[g][u];
-      }
-      l[g] = l[g] * alpha + ps;
-#pragma unroll
-      for (int e = 0; e < EPL; ++e) acc[g][e] *= alpha;
-    }
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      float vf[EPL];
-      E::unpack(vreg[u], vf);
-#pragma unroll
-      for (int g = 0; g < G; ++g) {
-#pragma unroll
-        for (int e = 0; e < EPL; ++e) acc[g][e] = fmaf(s[g][u], vf[e], acc[g][e]);
+        int t = c0 + u * RPW + grp;
+        if (t >= t1) t = t1 - 1;
+        int64_t blk;
+        int off;
+        a.pd.split(t, blk, off);
+        const int64_t slot = static_cast<int64_t>(s_pages[blk - blk0]) * a.pd.page_size + off;
+        kreg[u] = stream_load(kbase + slot * ROWB);
+        vreg[u] = stream_load(vbase + slot * ROWB);
       }
     }
+    if (c0 + CH <= t1)
+      fold_rows<E, TPR, G, U, RPW, false>(kreg, vreg, q, a.qscale, c0 + grp, t1, m, l, acc);
+    else
+      fold_rows<E, TPR, G, U, RPW, true>(kreg, vreg, q, a.qscale, c0 + grp, t1, m, l, acc);
   }
 
   // combine the lane groups of this wavefront
@@ -360,10 +426,19 @@ __global__ __launch_bounds__(64) void paged_decode_merge_kernel(const DecodeArgs
 template <typename E, int D, int G>
 void launch_decode(const DecodeArgs& a, int B, hipStream_t st) {
   dim3 grid(a.n_splits, a.Hc, B);
+  // rows per wavefront iteration: 8 loads of 64 / (D * elem / 16) rows each
+  const int chunk_rows = 8 * 64 / (D * static_cast<int>(sizeof(typename E::type)) / 16);
+  const bool aligned = a.pd.shift >= 0 && a.pd.page_size % chunk_rows == 0;
   if (a.n_splits == 1) {
-    hipLaunchKernelGGL((paged_decode_kernel<E, D, G, true>), grid, dim3(kThreads), 0, st, a);
+    if (aligned)
+      hipLaunchKernelGGL((paged_decode_kernel<E, D, G, true, true>), grid, dim3(kThreads), 0, st, a);
+    else
+      hipLaunchKernelGGL((paged_decode_kernel<E, D, G, true, false>), grid, dim3(kThreads), 0, st, a);
   } else {
-    hipLaunchKernelGGL((paged_decode_kernel<E, D, G, false>), grid, dim3(kThreads), 0, st, a);
+    if (aligned)
+      hipLaunchKernelGGL((paged_decode_kernel<E, D, G, false, true>), grid, dim3(kThreads), 0, st, a);
+    else
+      hipLaunchKernelGGL((paged_decode_kernel<E, D, G, false, false>), grid, dim3(kThreads), 0, st, a);
     hipLaunchKernelGGL((paged_decode_merge_kernel<E, D>), dim3(a.Hq, B), dim3(64), 0, st, a);
   }
 }
@@ -461,7 +536,7 @@ extern "C" int fp_paged_decode(const void* q, int64_t q_stride_b, int64_t q_stri
                page_table, pt_row_stride, batch_idx, input_pos, pos_index_type == FP_INDEX_I64,
                static_cast<char*>(out), out_stride_b * eb, out_stride_h * eb, lse,
                nullptr, nullptr, Hq, Hc, fp::PageDiv(page_size), n_pages, max_batch, n_slots,
-               max_context, split_tokens, ns, scale * kLog2e};
+               max_context, split_tokens, ns, scale * kLog2e};  // scores are kept in log2 units
   if (ns > 1) {
     const int64_t need = static_cast<int64_t>(B) * Hq * ns * (D + 2) * static_cast<int64_t>(sizeof(float));
     if (!workspace || workspace_bytes < need || !fp::aligned(workspace, 16))
