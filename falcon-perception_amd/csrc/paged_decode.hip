@@ -7,7 +7,7 @@
 // page_table[batch_idx[b], t / P] itself and bounds the context by input_pos[b].
 //
 // HBM-bound: every cached K and V row of every sequence is read exactly once.
-//   grid  = (splits, cache heads, batch); a workgroup of 4 wavefronts owns one
+//   grid  = (cache heads, batch, splits); a workgroup of 4 wavefronts owns one
 //           (sequence, cache head, token range) and serves all G = Hq / Hc query
 //           heads of that cache head from a single read of K and V.
 //   loads = a row (D elements) is covered by TPR = D * elem / 16 lanes holding
@@ -240,9 +240,12 @@ __global__ __launch_bounds__(kThreads) void paged_decode_kernel(const DecodeArgs
   __shared__ float s_acc[kWaves][G][D];
   __shared__ float s_ml[kWaves][G][2];
 
-  const int split = blockIdx.x;
-  const int hc = blockIdx.y;
-  const int b = blockIdx.z;
+  // Workgroups are dealt to the 8 XCDs round-robin by linear id.  Heads run fastest:
+  // every head of a sequence has the same amount of work, so each XCD gets an equal
+  // share of the non-empty workgroups whatever the context lengths are.
+  const int hc = blockIdx.x;
+  const int b = blockIdx.y;
+  const int split = blockIdx.z;
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
@@ -425,7 +428,7 @@ __global__ __launch_bounds__(64) void paged_decode_merge_kernel(const DecodeArgs
 
 template <typename E, int D, int G>
 void launch_decode(const DecodeArgs& a, int B, hipStream_t st) {
-  dim3 grid(a.n_splits, a.Hc, B);
+  dim3 grid(a.Hc, B, a.n_splits);
   // rows per wavefront iteration: 8 loads of 64 / (D * elem / 16) rows each
   const int chunk_rows = 8 * 64 / (D * static_cast<int>(sizeof(typename E::type)) / 16);
   const bool aligned = a.pd.shift >= 0 && a.pd.page_size % chunk_rows == 0;
