@@ -159,6 +159,109 @@ def make_decode_case(name: str, device="cuda", hbm_budget_gb: float | None = Non
     return case
 
 
+PREFILL_WORKLOADS = {
+    # BASELINE.json configs[2]: image prefix already paged, 512-token causal text chunk per sequence
+    "cfg3": dict(seed=3, dtype="bf16", n_seq=8, Hq=16, Hc=8, D=128, P=128, prefix_lo=256, prefix_hi=4096, chunk=512),
+    # whole sequences in one step (prefix 0): the image span rows are bidirectional
+    "cfg3w": dict(seed=3, dtype="bf16", n_seq=8, Hq=16, Hc=8, D=128, P=128, prefix_lo=256, prefix_hi=4096, chunk=512,
+                  whole=True),
+}
+
+
+@dataclass
+class PrefillCase:
+    """One chunked-prefill step's operands, all on the device."""
+
+    name: str
+    cfg: dict
+    cache: object
+    slots: list
+    prefixes: list
+    batch_idx: torch.Tensor   # [1, Lq] int64
+    input_pos: torch.Tensor   # [1, Lq] int64
+    row_limit: torch.Tensor   # [Lq] int32
+    q: torch.Tensor
+    k_new: torch.Tensor
+    v_new: torch.Tensor
+    pairs: int                # allowed (q, kv) pairs per head
+
+    @property
+    def page_size(self):
+        return self.cache.page_size
+
+    @property
+    def page_table(self):
+        return self.cache.page_table
+
+    @property
+    def pool_k(self):
+        return self.cache.kv_cache[0, 0, 0]
+
+    @property
+    def pool_v(self):
+        return self.cache.kv_cache[0, 1, 0]
+
+    def append(self):
+        self.cache.insert_kv(0, self.k_new, self.v_new, input_pos=self.input_pos, batch_idx=self.batch_idx)
+
+    def attend(self):
+        from falcon_perception_amd import ops
+
+        return ops.paged_prefill(self.q, self.pool_k, self.pool_v, self.cache.page_table, self.batch_idx,
+                                 self.row_limit, self.page_size)
+
+    def run(self):
+        self.append()
+        return self.attend()
+
+    def flops(self):
+        return 4 * self.cfg["D"] * self.cfg["Hq"] * self.pairs
+
+
+def make_prefill_case(name: str, device="cuda") -> PrefillCase:
+    from falcon_perception_amd.paged_attention import PagedKVCache
+
+    c = dict(PREFILL_WORKLOADS[name])
+    dtype = DTYPES[c["dtype"]]
+    gen = torch.Generator().manual_seed(c["seed"])
+    P, chunk, n_seq = c["P"], c["chunk"], c["n_seq"]
+    prefixes = [int(x) for x in torch.randint(c["prefix_lo"], c["prefix_hi"] + 1, (n_seq,), generator=gen)]
+    n_pages = sum(math.ceil((p + chunk) / P) for p in prefixes) + 64
+    cache = PagedKVCache(n_pages, P, n_seq + 1, c["Hc"], c["D"], 1, dtype, device=device)
+    cache.free_pages = (torch.randperm(n_pages - 1, generator=gen) + 1).tolist()
+    slots = []
+    for p in prefixes:
+        b = cache.allocate()
+        cache.reserve(b, torch.tensor([b], device=device), p + chunk)
+        slots.append(b)
+    dgen = torch.Generator(device=device).manual_seed(c["seed"])
+    cache.kv_cache.view(-1).normal_(generator=dgen)
+    whole = c.get("whole", False)
+    bidx, pos, lim, pairs = [], [], [], 0
+    for b, p in zip(slots, prefixes):
+        if whole:  # all p + chunk rows in this step; rows of the image span [0, p) see the whole span
+            n = p + chunk
+            row_pos = list(range(n))
+            row_lim = [max(t + 1, p) if t < p else t + 1 for t in range(n)]
+        else:      # only the chunk's rows; prefix already cached
+            n = chunk
+            row_pos = list(range(p, p + chunk))
+            row_lim = [t + 1 for t in row_pos]
+        gap = (-n) % 128
+        bidx += [b] * n + [0] * gap
+        pos += row_pos + [0] * gap
+        lim += row_lim + [0] * gap
+        pairs += sum(row_lim)
+    Lq = len(bidx)
+    q = torch.randn((1, c["Hq"], Lq, c["D"]), generator=dgen, device=device, dtype=torch.float32).to(dtype)
+    k_new = torch.randn((1, c["Hc"], Lq, c["D"]), generator=dgen, device=device, dtype=torch.float32).to(dtype)
+    v_new = torch.randn((1, c["Hc"], Lq, c["D"]), generator=dgen, device=device, dtype=torch.float32).to(dtype)
+    return PrefillCase(name, c, cache, slots, prefixes,
+                       torch.tensor([bidx], dtype=torch.int64, device=device),
+                       torch.tensor([pos], dtype=torch.int64, device=device),
+                       torch.tensor(lim, dtype=torch.int32, device=device), q, k_new, v_new, pairs)
+
+
 # --------------------------------------------------------------------------
 # timing
 # --------------------------------------------------------------------------

@@ -49,7 +49,7 @@ SIGNATURES = {
     "fp_hybrid_row_limits": (c_int, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_void_p]),
     "fp_paged_prefill": (c_int, [
         c_void_p, c_int64, c_int64, c_void_p, c_void_p,
-        c_void_p, c_int64, c_void_p, c_void_p, c_void_p,
+        c_void_p, c_int64, c_void_p, c_void_p,
         c_void_p, c_int64, c_int64, c_void_p,
         c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
         c_int64, c_float, c_int, c_void_p]),

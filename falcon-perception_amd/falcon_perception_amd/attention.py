@@ -210,7 +210,7 @@ def compiled_flex_attn_prefill(q: Tensor, k: Tensor, v: Tensor, score_mod=None, 
     pool_k = cache.kv_cache[step.layer_id, 0, 0]
     pool_v = cache.kv_cache[step.layer_id, 1, 0]
     out, lse = ops.paged_prefill(
-        q, pool_k, pool_v, cache.page_table, step.batch_idx, step.input_pos,
+        q, pool_k, pool_v, cache.page_table, step.batch_idx,
         block_mask.row_limit(step.input_pos), cache.page_size, scale=scale,
     )
     return _result(out, lse, return_aux, return_lse)

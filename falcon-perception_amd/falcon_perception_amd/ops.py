@@ -156,10 +156,11 @@ def hybrid_row_limits(input_ids: Tensor, soi_id: int, eoi_id: int) -> Tensor:
 
 
 def paged_prefill(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor, batch_idx: Tensor,
-                  input_pos: Tensor, row_limit: Tensor, page_size: int, *, scale: float | None = None,
+                  row_limit: Tensor, page_size: int, *, scale: float | None = None,
                   out: Tensor | None = None, lse: Tensor | None = None) -> tuple[Tensor, Tensor]:
-    """Chunked-prefill attention over the paged cache.  q [1, Hq, Lq, D]; returns out like q, lse [1, Hq, Lq]."""
-    N.require_cuda(q, pool_k, pool_v, page_table, batch_idx, input_pos, row_limit, out, lse)
+    """Chunked-prefill attention over the paged cache.  q [1, Hq, Lq, D]; row r sees keys
+    0..row_limit[r]-1 of sequence batch_idx[r]; returns out like q, lse [1, Hq, Lq]."""
+    N.require_cuda(q, pool_k, pool_v, page_table, batch_idx, row_limit, out, lse)
     one, Hq, Lq, D = q.shape
     if one != 1:
         raise RuntimeError("paged_prefill takes the packed layout [1, Hq, Lq, D]")
@@ -168,10 +169,11 @@ def paged_prefill(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor,
         raise RuntimeError("q / pool shape or dtype mismatch")
     q = _rows(q)
     batch_idx = batch_idx.reshape(-1).contiguous()
-    input_pos = input_pos.reshape(-1).contiguous()
     row_limit = row_limit.reshape(-1).contiguous()
-    if batch_idx.dtype != torch.int64 or input_pos.dtype != torch.int64 or row_limit.dtype != torch.int32:
-        raise RuntimeError("batch_idx, input_pos must be int64 and row_limit int32")
+    if batch_idx.dtype != torch.int64 or row_limit.dtype != torch.int32:
+        raise RuntimeError("batch_idx must be int64 and row_limit int32")
+    if batch_idx.shape[0] != Lq or row_limit.shape[0] != Lq:
+        raise RuntimeError("batch_idx and row_limit need one entry per query row")
     if scale is None:
         scale = 1.0 / math.sqrt(D)
     if out is None:
@@ -182,7 +184,7 @@ def paged_prefill(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor,
         raise RuntimeError("out rows must be dense and lse contiguous")
     rc = N.lib().fp_paged_prefill(
         q.data_ptr(), q.stride(2), q.stride(1), pool_k.data_ptr(), pool_v.data_ptr(),
-        page_table.data_ptr(), page_table.stride(0), batch_idx.data_ptr(), input_pos.data_ptr(),
+        page_table.data_ptr(), page_table.stride(0), batch_idx.data_ptr(),
         row_limit.data_ptr(), out.data_ptr(), out.stride(2), out.stride(1), lse.data_ptr(),
         Lq, Hq, Hc, D, page_size, page_table.shape[1], page_table.shape[0], n_slots,
         scale, N.dtype_code(q.dtype), N.stream_ptr(q.device))

@@ -189,15 +189,15 @@ int fp_hybrid_row_limits(const int64_t* input_ids, int32_t L,
  *
  *   q          [Lq, Hq, D] view with element strides (row, head) of the packed rows
  *   batch_idx  [Lq] int64 cache slot of each row (0 = padding: out 0, lse -inf)
- *   input_pos  [Lq] int64 logical position of each row in its sequence
  *   row_limit  [Lq] int32 logical keys 0..row_limit-1 of the row's sequence are visible
+ *              (row position + 1 for a causal row, the end of the image span inside one);
+ *              every such key must already be in the pages
  *   out        [Lq, Hq, D] view, strides (row, head); lse [Hq, Lq] float32
  */
 int fp_paged_prefill(const void* q, int64_t q_stride_row, int64_t q_stride_h,
                      const void* pool_k, const void* pool_v,
                      const int64_t* page_table, int64_t pt_row_stride,
-                     const int64_t* batch_idx, const int64_t* input_pos,
-                     const int32_t* row_limit,
+                     const int64_t* batch_idx, const int32_t* row_limit,
                      void* out, int64_t out_stride_row, int64_t out_stride_h,
                      float* lse,
                      int32_t Lq, int32_t Hq, int32_t Hc, int32_t D,

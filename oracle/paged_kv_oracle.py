@@ -399,8 +399,8 @@ def prefill_attention_paged(q, pool_k, pool_v, page_table, batch_idx, input_pos,
     """Chunked prefill over the paged cache, float64.
 
     q [1, Hq, Lq, D] packed query rows; row r belongs to cache slot
-    batch_idx[r] at logical position input_pos[r] and sees logical keys
-    0 .. row_limit[r]-1 of its own sequence (row_limit = max(pos + 1, image-span
+    batch_idx[r] (its position input_pos[r] enters only through row_limit and may be
+    None) and sees logical keys 0 .. row_limit[r]-1 of its own sequence (row_limit = max(pos + 1, image-span
     end): bidirectional inside the image span, causal elsewhere,
     attention.py:75-96), read from pages.  Rows with batch_idx 0 are padding:
     out 0, lse -inf.
@@ -422,8 +422,6 @@ def prefill_attention_paged(q, pool_k, pool_v, page_table, batch_idx, input_pos,
         n = int(lim[r])
         if b == 0 or n <= 0:
             continue
-        t = np.arange(n)
-        slots = pt[b, t // page_size] * page_size + t % page_size
         for h in range(Hq):
             g = h // G
             key = (b, g)
@@ -436,5 +434,4 @@ def prefill_attention_paged(q, pool_k, pool_v, page_table, batch_idx, input_pos,
             K, V = cache[key]
             s = (K[:n] @ q[0, h, r]) * scale
             out[0, h, r], lse[0, h, r] = _softmax_av(s, V[:n])
-        del slots
     return out, lse

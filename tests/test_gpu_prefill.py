@@ -1,0 +1,164 @@
+"""GPU parity: MFMA chunked-prefill attention over the paged cache under the hybrid mask,
+against the float64 oracle.  Tolerance (north star): 2e-2 absolute / 1e-2 relative in bf16."""
+
+import numpy as np
+import pytest
+import torch
+from torch.nn.attention.flex_attention import AuxRequest
+
+from falcon_perception_amd import attention as A
+from falcon_perception_amd import ops
+from oracle import paged_kv_oracle as O
+from tests.gpu_cases import DEV, PagedState, f64, randn
+from tests.test_oracle_masks import EOI, IMG, PAD, SOI, TXT, packed_case
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.bfloat16: (2e-2, 1e-2), torch.float16: (4e-3, 4e-3)}
+
+
+def assert_close(out, lse, eo, el, dtype, rows=None):
+    atol, rtol = TOL[dtype]
+    go, gl = f64(out), f64(lse)
+    if rows is not None:
+        go, gl, eo, el = go[:, :, rows], gl[:, :, rows], eo[:, :, rows], el[:, :, rows]
+    np.testing.assert_allclose(go, eo, atol=atol, rtol=rtol)
+    np.testing.assert_allclose(gl, el, atol=max(atol * 0.1, 1e-4), rtol=rtol)
+
+
+def prefill_through_api(st, ids, bidx, pos, Hq, dtype, pad_to):
+    """insert_kv + compiled_flex_attn_prefill exactly as model.py:150-162 calls them."""
+    cache = st.cache
+    L = len(ids)
+    t_ids = torch.from_numpy(ids)[None].to(DEV)
+    t_b = torch.from_numpy(bidx)[None].to(DEV)
+    t_p = torch.from_numpy(pos)[None].to(DEV)
+    mask = cache.create_prefill_blockmask(t_b, t_ids, SOI, EOI)
+    k = randn(st.gen, (1, st.Hc, L, st.D), dtype)
+    v = randn(st.gen, (1, st.Hc, L, st.D), dtype)
+    q = randn(st.gen, (1, Hq, L, st.D), dtype)
+    K, V = cache.insert_kv(0, k.to(DEV), v.to(DEV), input_pos=t_p, batch_idx=t_b)
+    out, aux = A.compiled_flex_attn_prefill(q.to(DEV), K, V, block_mask=mask, return_aux=AuxRequest(lse=True),
+                                            kernel_options={"FORCE_USE_FLEX_ATTENTION": True})
+    return q, k, v, out, aux.lse
+
+
+def layout_for(sizes):
+    """One sequence per entry: (slot, text before, image tokens, text after)."""
+    return [(slot, ([("t", a)] if a else []) + ([("i", n)] if n else []) + ([("t", b)] if b else []))
+            for slot, a, n, b in sizes]
+
+
+def repack(layout, pad_to):
+    ids, bidx, pos = [], [], []
+    for slot, segs in layout:
+        start = len(ids)
+        for kind, n in segs:
+            ids += [TXT] * n if kind == "t" else [SOI] + [IMG + 1] * 4 + [IMG] * n + [EOI]
+        L = len(ids) - start
+        bidx += [slot] * L
+        pos += list(range(L))
+        gap = (-L) % pad_to
+        ids += [PAD] * gap
+        bidx += [0] * gap
+        pos += [0] * gap
+    return np.array(ids), np.array(bidx), np.array(pos)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)
+@pytest.mark.parametrize("D,G", [(128, 1), (128, 2), (64, 4)])
+def test_whole_sequence_prefill_matches_the_reference_semantics(dtype, D, G):
+    """The reference's own prefill (packed sequences, each padded to 128): attention over the packed
+    fresh K/V under image-prefix OR document-causal (paged_attention.py:343-393)."""
+    Hc = 2
+    layout = layout_for([(1, 5, 150, 40), (2, 0, 60, 200), (3, 131, 0, 0)])
+    ids, bidx, pos = repack(layout, 128)
+    st = PagedState(1, n_pages=64, page_size=64, max_batch=6, Hc=Hc, D=D, dtype=dtype)
+    for slot in (1, 2, 3):
+        st.add_sequence(int((bidx == slot).sum()))
+    q, k, v, out, lse = prefill_through_api(st, ids, bidx, pos, Hc * G, dtype, 128)
+    eo, el = O.prefill_attention_packed(f64(q), f64(k), f64(v), bidx[None], ids[None], SOI, EOI)
+    real = np.flatnonzero(bidx != 0)
+    assert_close(out, lse, eo, el, dtype, rows=real)
+    pad = np.flatnonzero(bidx == 0)
+    assert not f64(out)[:, :, pad].any() and np.isneginf(f64(lse)[:, :, pad]).all()
+
+
+def test_unaligned_packing_and_small_pages():
+    """Sequences packed back to back without padding (several sequences per 128-row tile), page size 16."""
+    dtype = torch.bfloat16
+    layout = layout_for([(1, 3, 20, 30), (2, 10, 0, 0), (3, 0, 40, 9), (4, 77, 0, 0), (5, 1, 0, 0)])
+    ids, bidx, pos = repack(layout, 1)
+    st = PagedState(2, n_pages=40, page_size=16, max_batch=8, Hc=2, D=128, dtype=dtype)
+    for slot in (1, 2, 3, 4, 5):
+        st.add_sequence(int((bidx == slot).sum()))
+    q, k, v, out, lse = prefill_through_api(st, ids, bidx, pos, 4, dtype, 1)
+    eo, el = O.prefill_attention_packed(f64(q), f64(k), f64(v), bidx[None], ids[None], SOI, EOI)
+    assert_close(out, lse, eo, el, dtype)
+
+
+@pytest.mark.parametrize("prefix,chunk", [(300, 100), (128, 128), (1000, 37), (0, 200)])
+def test_chunk_over_a_paged_prefix(prefix, chunk):
+    """Chunked prefill: the prefix (image span + text) is already in pages, the chunk's rows attend
+    over prefix + chunk; equals the chunk's rows of the whole-sequence result."""
+    dtype = torch.bfloat16
+    Hc, G, D, P = 2, 2, 128, 64
+    total = prefix + chunk
+    n_img = max(0, min(prefix - 10, 200))
+    ids = np.array(([TXT] * 2 + [SOI] + [IMG] * n_img + [EOI] if n_img else []) + [TXT] * total)[:total]
+    st = PagedState(3, n_pages=40, page_size=P, max_batch=4, Hc=Hc, D=D, dtype=dtype)
+    b = st.add_sequence(total)
+    bidx = np.full(total, b)
+    pos = np.arange(total)
+    k = randn(st.gen, (1, Hc, total, D), dtype)
+    v = randn(st.gen, (1, Hc, total, D), dtype)
+    q = randn(st.gen, (1, Hc * G, total, D), dtype)
+    cache = st.cache
+    dev = lambda a: torch.from_numpy(a)[None].to(DEV)
+    if prefix:
+        cache.insert_kv(0, k[:, :, :prefix].to(DEV), v[:, :, :prefix].to(DEV), input_pos=dev(pos[:prefix]),
+                        batch_idx=dev(bidx[:prefix]))
+    # the chunk step: mask from the chunk's own tokens, positions continue after the prefix
+    mask = cache.create_prefill_blockmask(dev(bidx[prefix:]), dev(ids[prefix:]), SOI, EOI)
+    K, V = cache.insert_kv(0, k[:, :, prefix:].to(DEV), v[:, :, prefix:].to(DEV), input_pos=dev(pos[prefix:]),
+                           batch_idx=dev(bidx[prefix:]))
+    out, aux = A.compiled_flex_attn_prefill(q[:, :, prefix:].to(DEV), K, V, block_mask=mask,
+                                            return_aux=AuxRequest(lse=True))
+    eo, el = O.prefill_attention_packed(f64(q), f64(k), f64(v), bidx[None], ids[None], SOI, EOI)
+    assert_close(out, aux.lse, eo[:, :, prefix:], el[:, :, prefix:], dtype)
+
+
+def test_row_limits_direct_and_empty_rows():
+    """ops.paged_prefill with explicit limits: limit 0 gives out 0 / lse -inf; limits beyond the row's
+    own position give bidirectional attention."""
+    dtype = torch.bfloat16
+    st = PagedState(4, n_pages=16, page_size=32, max_batch=4, Hc=1, D=64, dtype=dtype)
+    b = st.add_sequence(150)
+    k, v, bt, pt, _, _ = st.prefill_random()
+    q = randn(st.gen, (1, 2, 150, 64), dtype)
+    lim = torch.randint(0, 151, (150,), generator=st.gen, dtype=torch.int32)
+    lim[:5] = 0
+    bidx = torch.full((150,), b, dtype=torch.int64)
+    pk, pv = st.pool_planes()
+    out, lse = ops.paged_prefill(q.to(DEV), pk, pv, st.cache.page_table, bidx.to(DEV), lim.to(DEV), st.P)
+    eo, el = O.prefill_attention_paged(f64(q), f64(pk), f64(pv), st.mirror.page_table, bidx.numpy(),
+                                       np.arange(150), lim.numpy(), st.P)
+    assert_close(out, lse, eo, el, dtype)
+    assert not f64(out)[:, :, :5].any() and np.isneginf(f64(lse)[:, :, :5]).all()
+
+
+def test_cfg3_chunked_prefill_shape():
+    """BASELINE configs[2]: 8 sequences, image prefix U[256,4096] already paged, 512-token text chunk each,
+    16 q / 8 kv heads, D 128, page 128.  Checked on the first and last sequences (the oracle is O(L^2))."""
+    import bench
+
+    case = bench.make_prefill_case("cfg3", device=DEV)
+    out, lse = case.run()
+    pk, pv = case.pool_k.float().cpu().numpy(), case.pool_v.float().cpu().numpy()
+    bidx = case.batch_idx.cpu().numpy().reshape(-1)
+    lim = case.row_limit.cpu().numpy()
+    for s in (0, len(case.slots) - 1):
+        rows = np.flatnonzero(bidx == case.slots[s])[::7]  # every 7th row of the chunk
+        eo, el = O.prefill_attention_paged(f64(case.q[:, :, rows]), pk, pv, case.page_table.cpu().numpy(),
+                                           bidx[rows], None, lim[rows], case.page_size)
+        assert_close(out[:, :, rows], lse[:, :, rows], eo, el, torch.bfloat16)
