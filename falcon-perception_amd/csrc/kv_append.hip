@@ -10,9 +10,15 @@
 // of one head, so a wavefront writes consecutive slots of a page as one
 // contiguous run and reads whole 256-byte rows of the source.  The slot is
 // computed in the kernel from the page table, there is no separate slot-mapping pass.
+// Loads and stores are non-temporal: the rows are touched once and should not displace
+// cache lines other kernels reuse.
 #include "fp_common.h"
 
 namespace {
+
+// clang vector types: the non-temporal load/store builtins take these, not HIP's uint4
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+typedef uint32_t v2u __attribute__((ext_vector_type(2)));
 
 struct AppendArgs {
   char* pool_k;
@@ -63,8 +69,8 @@ __global__ __launch_bounds__(kThreads) void kv_append_kernel(const AppendArgs a)
     }
     const int64_t ko = t * a.ks_t + h * a.ks_h + s * a.ks_s + static_cast<int64_t>(c) * sizeof(Vec);
     const int64_t vo = t * a.vs_t + h * a.vs_h + s * a.vs_s + static_cast<int64_t>(c) * sizeof(Vec);
-    kreg[j] = *reinterpret_cast<const Vec*>(a.k + ko);
-    vreg[j] = *reinterpret_cast<const Vec*>(a.v + vo);
+    kreg[j] = __builtin_nontemporal_load(reinterpret_cast<const Vec*>(a.k + ko));
+    vreg[j] = __builtin_nontemporal_load(reinterpret_cast<const Vec*>(a.v + vo));
 
     const int64_t b = a.batch_idx[t];
     const int64_t pos = fp::load_index(a.input_pos, tok, a.pos_i64);
@@ -84,8 +90,8 @@ __global__ __launch_bounds__(kThreads) void kv_append_kernel(const AppendArgs a)
 #pragma unroll
   for (int j = 0; j < kItems; ++j) {
     if (dst[j] < 0) continue;
-    *reinterpret_cast<Vec*>(a.pool_k + dst[j]) = kreg[j];
-    *reinterpret_cast<Vec*>(a.pool_v + dst[j]) = vreg[j];
+    __builtin_nontemporal_store(kreg[j], reinterpret_cast<Vec*>(a.pool_k + dst[j]));
+    __builtin_nontemporal_store(vreg[j], reinterpret_cast<Vec*>(a.pool_v + dst[j]));
   }
 }
 
@@ -143,8 +149,8 @@ extern "C" int fp_kv_append(void* pool_k, void* pool_v, const void* k, const voi
 
   hipStream_t st = static_cast<hipStream_t>(stream);
   switch (vec) {
-    case 16: launch<uint4>(a, H, st); break;
-    case 8: launch<uint2>(a, H, st); break;
+    case 16: launch<v4u>(a, H, st); break;
+    case 8: launch<v2u>(a, H, st); break;
     case 4: launch<uint32_t>(a, H, st); break;
     default: launch<uint16_t>(a, H, st); break;
   }

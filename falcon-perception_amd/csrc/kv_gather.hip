@@ -15,6 +15,9 @@
 
 namespace {
 
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+typedef uint32_t v2u __attribute__((ext_vector_type(2)));
+
 struct GatherArgs {
   const char* pool;
   char* out;
@@ -54,7 +57,7 @@ __global__ __launch_bounds__(kThreads) void kv_gather_kernel(const GatherArgs a)
   for (int j = 0; j < kItems; ++j) {
     const int64_t i = base + static_cast<int64_t>(j) * kThreads;
     dst[j] = -1;
-    reg[j] = Vec{};
+    reg[j] = Vec(0);
     if (i >= items) continue;
     const int t = static_cast<int>(i / a.chunks);
     const int c = static_cast<int>(i - static_cast<int64_t>(t) * a.chunks);
@@ -68,12 +71,12 @@ __global__ __launch_bounds__(kThreads) void kv_gather_kernel(const GatherArgs a)
     const int64_t slot = page * a.pd.page_size + off;
     if (slot < 0 || slot >= a.n_slots) continue;
     const int64_t src = (static_cast<int64_t>(h) * a.n_slots + slot) * a.row_bytes + static_cast<int64_t>(c) * sizeof(Vec);
-    reg[j] = *reinterpret_cast<const Vec*>(a.pool + src);
+    reg[j] = __builtin_nontemporal_load(reinterpret_cast<const Vec*>(a.pool + src));
   }
 #pragma unroll
   for (int j = 0; j < kItems; ++j) {
     if (dst[j] < 0) continue;
-    *reinterpret_cast<Vec*>(a.out + dst[j]) = reg[j];
+    __builtin_nontemporal_store(reg[j], reinterpret_cast<Vec*>(a.out + dst[j]));
   }
 }
 
@@ -140,8 +143,8 @@ extern "C" int fp_kv_gather(const void* pool, void* out, int64_t out_stride_b, i
 
   hipStream_t st = static_cast<hipStream_t>(stream);
   switch (vec) {
-    case 16: launch_gather<uint4>(a, B, H, st); break;
-    case 8: launch_gather<uint2>(a, B, H, st); break;
+    case 16: launch_gather<v4u>(a, B, H, st); break;
+    case 8: launch_gather<v2u>(a, B, H, st); break;
     case 4: launch_gather<uint32_t>(a, B, H, st); break;
     default: launch_gather<uint16_t>(a, B, H, st); break;
   }
