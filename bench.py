@@ -30,6 +30,7 @@ for _p in (ROOT, os.path.join(ROOT, "falcon-perception_amd")):
 import torch  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, published peak
 MODEL_LAYERS = 28       # Falcon Perception 0.6B (reference __init__.py:36)
 
 # name -> shape of the decode workloads of BASELINE.json (configs[0], [1], [3] decode part, [4])
@@ -41,6 +42,10 @@ DECODE_WORKLOADS = {
     "cfg5": dict(seed=5, dtype="bf16", B=256, Hq=32, Hc=8, D=128, P=128, n_pages=None, prefix=4096, lo=256, hi=12288),
 }
 DTYPES = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
+
+# HBM bytes per launch of paged_decode_kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# (profiles/), scaled by the same counters on a plain copy of known size; None = not measured
+TRAFFIC_BYTES = {}
 
 
 @dataclass
@@ -85,13 +90,13 @@ class DecodeCase:
         ops.kv_append(self.pool_k, self.pool_v, self.k_new, self.v_new, self.cache.page_table,
                       self.batch_idx, self.input_pos.view(-1, 1), self.page_size, clamp_negative=True)
 
-    def attend(self):
+    def attend(self, phase="both"):
         from falcon_perception_amd import ops
 
         return ops.paged_decode(self.q, self.pool_k, self.pool_v, self.cache.page_table, self.batch_idx,
                                 self.input_pos, self.page_size, self.max_context,
                                 split_tokens=self.split_tokens, workspace=self.workspace,
-                                out=self.out, lse=self.lse)
+                                out=self.out, lse=self.lse, phase=phase)
 
     def run(self):
         self.append()
@@ -310,6 +315,66 @@ def graph_ms(fn, steps: int) -> float:
     return (time.perf_counter() - t0) * 1e3 / steps
 
 
+def append_gather_rates(steps: int = 20, T: int = 32768, H: int = 16, D: int = 128, P: int = 128) -> dict:
+    """KV append and page gather at a prefill-sized batch of tokens (the engine's prefill limit,
+    reference paged_inference.py:233): bf16, 16 stored heads, one fragmented page table."""
+    from falcon_perception_amd import ops
+    from falcon_perception_amd.paged_attention import PagedKVCache
+
+    dev, dtype = "cuda", torch.bfloat16
+    cache = PagedKVCache(T // P + 16, P, 4, H, D, 1, dtype, device=dev)
+    g = torch.Generator().manual_seed(7)
+    cache.free_pages = (torch.randperm(cache.n_pages - 1, generator=g) + 1).tolist()
+    b = cache.allocate()
+    cache.reserve(b, torch.tensor([b], device=dev), T)
+    # the model hands K/V over as [1, L, H, D] memory viewed as [1, H, L, D] (reference model.py:118-119)
+    k = torch.randn((1, T, H, D), device=dev, dtype=dtype).permute(0, 2, 1, 3)
+    v = torch.randn((1, T, H, D), device=dev, dtype=dtype).permute(0, 2, 1, 3)
+    bidx = torch.full((1, T), b, dtype=torch.int64, device=dev)
+    pos = torch.arange(T, dtype=torch.int64, device=dev)[None]
+    pk, pv = cache.kv_cache[0, 0, 0], cache.kv_cache[0, 1, 0]
+    k_rows, v_rows = k[0].transpose(0, 1).unsqueeze(2), v[0].transpose(0, 1).unsqueeze(2)
+    flat_b, flat_p = bidx.reshape(T), pos.reshape(T, 1)
+
+    def do_append():
+        ops.kv_append(pk, pv, k_rows, v_rows, cache.page_table, flat_b, flat_p, P, clamp_negative=False)
+
+    lens = torch.tensor([T], device=dev)
+    slots = torch.tensor([b], device=dev)
+    out = torch.empty((1, H, T, D), dtype=dtype, device=dev)
+
+    def do_gather():
+        ops.kv_gather(pk, cache.page_table, slots, lens, P, T, out=out)
+
+    for _ in range(3):
+        do_append()
+        do_gather()
+    ms_a = event_ms(do_append, steps)
+    ms_g = event_ms(do_gather, steps)
+    e = 2
+    bytes_a = 2 * T * (2 * H * D * e) + 8 * T
+    bytes_g = 2 * T * (H * D * e)
+    return {"tokens": T, "heads": H, "head_dim": D,
+            "kv_append_ms": ms_a, "kv_append_gbps": bytes_a / (ms_a * 1e-3) / 1e9,
+            "kv_append_frac_of_peak": bytes_a / (ms_a * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "kv_gather_ms": ms_g, "kv_gather_gbps": bytes_g / (ms_g * 1e-3) / 1e9,
+            "kv_gather_frac_of_peak": bytes_g / (ms_g * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+
+
+def prefill_rate(steps: int = 10) -> dict:
+    """Chunked prefill at BASELINE configs[2]: append the 512-token chunks, attend over the paged prefix."""
+    case = make_prefill_case("cfg3")
+    case.append()
+    for _ in range(3):
+        case.attend()
+    ms = event_ms(case.attend, steps)
+    ms_a = event_ms(case.append, steps)
+    tf = case.flops() / (ms * 1e-3) / 1e12
+    return {"workload": "cfg3: 8 sequences, paged prefix U[256,4096], 512-token chunk each, 16 q / 8 kv heads, D 128",
+            "paged_prefill_ms": ms, "tflops": tf, "frac_of_bf16_mfma_peak": tf / MFMA_BF16_PEAK_TFLOPS,
+            "chunk_append_ms": ms_a, "flops": case.flops()}
+
+
 def cpu_baseline(case: DecodeCase, budget_s: float = 20.0) -> dict:
     """The reference's op sequence for one decode layer-step, ported to torch-CPU, timed on the
     host cores on a batch subset sized to roughly `budget_s` seconds."""
@@ -361,6 +426,10 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="cfg2", choices=sorted(DECODE_WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--decode-only", action="store_true", help="skip the append/gather/prefill side measurements")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="also run a plain 1 GiB device copy a few times, so a rocprofv3 --pmc run of this "
+                         "command holds a kernel of known traffic next to the decode kernel")
     ap.add_argument("--hbm-budget-gb", type=float, default=None, help="pool size for cfg5")
     args = ap.parse_args()
 
@@ -378,16 +447,27 @@ def main() -> int:
     case = make_decode_case(args.workload, hbm_budget_gb=args.hbm_budget_gb)
     c = case.cfg
 
+    if args.pmc_calibration:
+        src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")  # 1 GiB read + 1 GiB written per copy
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     ms_step = time_steps(case.run, args.steps, args.warmup)
     ms_graph = graph_ms(case.run, args.steps)
     ms_decode = event_ms(case.attend, args.steps)
+    ms_partial = event_ms(lambda: case.attend("partial"), args.steps)  # the dominant kernel alone
+    ms_merge = event_ms(lambda: case.attend("merge"), args.steps)
     ms_append = event_ms(case.append, args.steps)
+    case.attend()
 
     alg_decode = case.bytes_decode()
     alg_append = case.bytes_append()
     alg_step = alg_decode + alg_append
     value = alg_step / (ms_step * 1e-3) / 1e9
-    achieved = alg_decode / (ms_decode * 1e-3) / 1e9
+    achieved = alg_decode / (ms_partial * 1e-3) / 1e9
 
     result = {
         "metric": "paged decode attn + KV append HBM GB/s (% of peak); decode tok/s",
@@ -403,12 +483,17 @@ def main() -> int:
         "decode_tok_s_model": c["B"] / (ms_step * 1e-3) / MODEL_LAYERS,
         "ms_per_step_hip_graph": ms_graph,
         "value_hip_graph": alg_step / (ms_graph * 1e-3) / 1e9,
-        "kernels": {"paged_decode_ms": ms_decode, "kv_append_ms": ms_append,
-                    "kv_append_gbps": alg_append / (ms_append * 1e-3) / 1e9},
-        "roofline": {"bound": "hbm", "kernel": "paged_decode_kernel (+ merge)", "achieved": achieved,
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
-                     "algorithmic_bytes": alg_decode},
+        "kernels": {"paged_decode_ms": ms_decode, "paged_decode_partial_ms": ms_partial,
+                    "paged_decode_merge_ms": ms_merge,
+                    "paged_decode_gbps": alg_decode / (ms_decode * 1e-3) / 1e9,
+                    "kv_append_ms": ms_append, "kv_append_gbps": alg_append / (ms_append * 1e-3) / 1e9},
+        "roofline": {"bound": "hbm", "kernel": "paged_decode_kernel", "achieved": achieved,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
+                     "traffic": TRAFFIC_BYTES.get(case.name), "algorithmic_bytes": alg_decode},
     }
+    if not args.decode_only:
+        result["prefill_sized"] = append_gather_rates()
+        result["chunked_prefill"] = prefill_rate()
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(case)
         result["gpu_over_cpu"] = value / result["cpu_baseline"]["value"]

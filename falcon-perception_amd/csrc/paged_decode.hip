@@ -426,42 +426,50 @@ __global__ __launch_bounds__(64) void paged_decode_merge_kernel(const DecodeArgs
     a.lse[static_cast<int64_t>(b) * a.Hq + hq] = ns > 0 ? (mn + log2f(den)) * kLn2 : -INFINITY;
 }
 
+constexpr int kPhasePartial = 1;
+constexpr int kPhaseMerge = 2;
+
 template <typename E, int D, int G>
-void launch_decode(const DecodeArgs& a, int B, hipStream_t st) {
+void launch_decode(const DecodeArgs& a, int B, int phases, hipStream_t st) {
   dim3 grid(a.Hc, B, a.n_splits);
   // rows per wavefront iteration: 8 loads of 64 / (D * elem / 16) rows each
   const int chunk_rows = 8 * 64 / (D * static_cast<int>(sizeof(typename E::type)) / 16);
   const bool aligned = a.pd.shift >= 0 && a.pd.page_size % chunk_rows == 0;
   if (a.n_splits == 1) {
+    // one split covers every context: the partial pass writes out and lse itself
+    if (!(phases & kPhasePartial)) return;
     if (aligned)
       hipLaunchKernelGGL((paged_decode_kernel<E, D, G, true, true>), grid, dim3(kThreads), 0, st, a);
     else
       hipLaunchKernelGGL((paged_decode_kernel<E, D, G, true, false>), grid, dim3(kThreads), 0, st, a);
   } else {
-    if (aligned)
-      hipLaunchKernelGGL((paged_decode_kernel<E, D, G, false, true>), grid, dim3(kThreads), 0, st, a);
-    else
-      hipLaunchKernelGGL((paged_decode_kernel<E, D, G, false, false>), grid, dim3(kThreads), 0, st, a);
-    hipLaunchKernelGGL((paged_decode_merge_kernel<E, D>), dim3(a.Hq, B), dim3(64), 0, st, a);
+    if (phases & kPhasePartial) {
+      if (aligned)
+        hipLaunchKernelGGL((paged_decode_kernel<E, D, G, false, true>), grid, dim3(kThreads), 0, st, a);
+      else
+        hipLaunchKernelGGL((paged_decode_kernel<E, D, G, false, false>), grid, dim3(kThreads), 0, st, a);
+    }
+    if (phases & kPhaseMerge)
+      hipLaunchKernelGGL((paged_decode_merge_kernel<E, D>), dim3(a.Hq, B), dim3(64), 0, st, a);
   }
 }
 
 template <typename E, int D>
-int dispatch_group(const DecodeArgs& a, int B, hipStream_t st) {
+int dispatch_group(const DecodeArgs& a, int B, int phases, hipStream_t st) {
   switch (a.Hq / a.Hc) {
-    case 1: launch_decode<E, D, 1>(a, B, st); return FP_OK;
-    case 2: launch_decode<E, D, 2>(a, B, st); return FP_OK;
-    case 4: launch_decode<E, D, 4>(a, B, st); return FP_OK;
-    case 8: launch_decode<E, D, 8>(a, B, st); return FP_OK;
+    case 1: launch_decode<E, D, 1>(a, B, phases, st); return FP_OK;
+    case 2: launch_decode<E, D, 2>(a, B, phases, st); return FP_OK;
+    case 4: launch_decode<E, D, 4>(a, B, phases, st); return FP_OK;
+    case 8: launch_decode<E, D, 8>(a, B, phases, st); return FP_OK;
     default: return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_decode: Hq/Hc = %d (supported: 1, 2, 4, 8)", a.Hq / a.Hc);
   }
 }
 
 template <typename E>
-int dispatch_dim(const DecodeArgs& a, int B, int D, hipStream_t st) {
+int dispatch_dim(const DecodeArgs& a, int B, int D, int phases, hipStream_t st) {
   switch (D) {
-    case 64: return dispatch_group<E, 64>(a, B, st);
-    case 128: return dispatch_group<E, 128>(a, B, st);
+    case 64: return dispatch_group<E, 64>(a, B, phases, st);
+    case 128: return dispatch_group<E, 128>(a, B, phases, st);
     default: return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_decode: head_dim %d (supported: 64, 128)", D);
   }
 }
@@ -496,14 +504,16 @@ extern "C" int64_t fp_paged_decode_workspace_bytes(int32_t B, int32_t Hq, int32_
   return static_cast<int64_t>(B) * Hq * ns * (D + 2) * static_cast<int64_t>(sizeof(float));
 }
 
-extern "C" int fp_paged_decode(const void* q, int64_t q_stride_b, int64_t q_stride_h, const void* pool_k,
-                               const void* pool_v, const int64_t* page_table, int64_t pt_row_stride,
-                               const int64_t* batch_idx, const void* input_pos, int pos_index_type,
-                               void* out, int64_t out_stride_b, int64_t out_stride_h, float* lse,
-                               void* workspace, int64_t workspace_bytes, int32_t B, int32_t Hq, int32_t Hc,
-                               int32_t D, int32_t page_size, int32_t n_pages, int32_t max_batch,
-                               int64_t n_slots, int32_t max_context, int32_t split_tokens, float scale,
-                               int dtype, void* stream) {
+namespace {
+
+int decode_entry(int phases, const void* q, int64_t q_stride_b, int64_t q_stride_h, const void* pool_k,
+                 const void* pool_v, const int64_t* page_table, int64_t pt_row_stride,
+                 const int64_t* batch_idx, const void* input_pos, int pos_index_type,
+                 void* out, int64_t out_stride_b, int64_t out_stride_h, float* lse,
+                 void* workspace, int64_t workspace_bytes, int32_t B, int32_t Hq, int32_t Hc,
+                 int32_t D, int32_t page_size, int32_t n_pages, int32_t max_batch,
+                 int64_t n_slots, int32_t max_context, int32_t split_tokens, float scale,
+                 int dtype, void* stream) {
   const int eb = fp::elem_bytes(dtype);
   if (eb == 0) return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_decode: unknown dtype %d", dtype);
   if (B < 0 || Hq <= 0 || Hc <= 0 || D <= 0 || page_size <= 0 || n_pages <= 0 || max_batch <= 0 ||
@@ -552,10 +562,28 @@ extern "C" int fp_paged_decode(const void* q, int64_t q_stride_b, int64_t q_stri
   hipStream_t st = static_cast<hipStream_t>(stream);
   int rc;
   switch (dtype) {
-    case FP_DTYPE_F32: rc = dispatch_dim<F32>(a, B, D, st); break;
-    case FP_DTYPE_BF16: rc = dispatch_dim<BF16>(a, B, D, st); break;
-    default: rc = dispatch_dim<F16>(a, B, D, st); break;
+    case FP_DTYPE_F32: rc = dispatch_dim<F32>(a, B, D, phases, st); break;
+    case FP_DTYPE_BF16: rc = dispatch_dim<BF16>(a, B, D, phases, st); break;
+    default: rc = dispatch_dim<F16>(a, B, D, phases, st); break;
   }
   if (rc != FP_OK) return rc;
   return fp::check_launch("fp_paged_decode");
 }
+
+}  // namespace
+
+#define FP_DECODE_PARAMS                                                                                   \
+  const void *q, int64_t q_stride_b, int64_t q_stride_h, const void *pool_k, const void *pool_v,          \
+      const int64_t *page_table, int64_t pt_row_stride, const int64_t *batch_idx, const void *input_pos,  \
+      int pos_index_type, void *out, int64_t out_stride_b, int64_t out_stride_h, float *lse,              \
+      void *workspace, int64_t workspace_bytes, int32_t B, int32_t Hq, int32_t Hc, int32_t D,             \
+      int32_t page_size, int32_t n_pages, int32_t max_batch, int64_t n_slots, int32_t max_context,        \
+      int32_t split_tokens, float scale, int dtype, void *stream
+#define FP_DECODE_ARGS                                                                                     \
+  q, q_stride_b, q_stride_h, pool_k, pool_v, page_table, pt_row_stride, batch_idx, input_pos,             \
+      pos_index_type, out, out_stride_b, out_stride_h, lse, workspace, workspace_bytes, B, Hq, Hc, D,     \
+      page_size, n_pages, max_batch, n_slots, max_context, split_tokens, scale, dtype, stream
+
+extern "C" int fp_paged_decode(FP_DECODE_PARAMS) { return decode_entry(kPhasePartial | kPhaseMerge, FP_DECODE_ARGS); }
+extern "C" int fp_paged_decode_partial(FP_DECODE_PARAMS) { return decode_entry(kPhasePartial, FP_DECODE_ARGS); }
+extern "C" int fp_paged_decode_merge(FP_DECODE_PARAMS) { return decode_entry(kPhaseMerge, FP_DECODE_ARGS); }

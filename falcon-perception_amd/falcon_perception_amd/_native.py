@@ -46,6 +46,8 @@ SIGNATURES = {
         c_void_p, c_int64,
         c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
         c_int64, c_int32, c_int32, c_float, c_int, c_void_p]),
+    "fp_paged_decode_partial": None,  # same signature as fp_paged_decode, filled in below
+    "fp_paged_decode_merge": None,
     "fp_hybrid_row_limits": (c_int, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_void_p]),
     "fp_paged_prefill": (c_int, [
         c_void_p, c_int64, c_int64, c_void_p, c_void_p,
@@ -54,6 +56,9 @@ SIGNATURES = {
         c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
         c_int64, c_float, c_int, c_void_p]),
 }
+
+SIGNATURES["fp_paged_decode_partial"] = SIGNATURES["fp_paged_decode"]
+SIGNATURES["fp_paged_decode_merge"] = SIGNATURES["fp_paged_decode"]
 
 _lib = None
 

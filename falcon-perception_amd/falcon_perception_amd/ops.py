@@ -104,8 +104,11 @@ def decode_workspace_bytes(B: int, Hq: int, D: int, max_context: int, split_toke
 def paged_decode(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor, batch_idx: Tensor,
                  input_pos: Tensor, page_size: int, max_context: int, *, scale: float | None = None,
                  split_tokens: int = 0, workspace: Tensor | None = None,
-                 out: Tensor | None = None, lse: Tensor | None = None) -> tuple[Tensor, Tensor]:
-    """Single-query paged attention.  q [B, Hq, 1, D]; pools [Hc, N, D]; returns out [B, Hq, 1, D], lse [B, Hq, 1]."""
+                 out: Tensor | None = None, lse: Tensor | None = None, phase: str = "both") -> tuple[Tensor, Tensor]:
+    """Single-query paged attention.  q [B, Hq, 1, D]; pools [Hc, N, D]; returns out [B, Hq, 1, D], lse [B, Hq, 1].
+
+    `phase` = "both" (default), "partial" (split-K pass only, results stay in `workspace`) or
+    "merge" (cross-split merge of a previous partial pass with the same arguments)."""
     N.require_cuda(q, pool_k, pool_v, page_table, batch_idx, input_pos, workspace, out, lse)
     B, Hq, Sq, D = q.shape
     if Sq != 1:
@@ -129,7 +132,8 @@ def paged_decode(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor, 
         lse = torch.empty((B, Hq, 1), dtype=torch.float32, device=q.device)
     if out.stride(3) != 1 or not lse.is_contiguous() or lse.dtype != torch.float32:
         raise RuntimeError("out rows must be dense and lse contiguous float32")
-    rc = N.lib().fp_paged_decode(
+    entry = {"both": "fp_paged_decode", "partial": "fp_paged_decode_partial", "merge": "fp_paged_decode_merge"}[phase]
+    rc = getattr(N.lib(), entry)(
         q.data_ptr(), q.stride(0), q.stride(1), pool_k.data_ptr(), pool_v.data_ptr(),
         page_table.data_ptr(), page_table.stride(0), batch_idx.data_ptr(),
         input_pos.data_ptr(), N.index_code(input_pos),
@@ -138,7 +142,7 @@ def paged_decode(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor, 
         workspace.numel() * workspace.element_size() if workspace is not None else 0,
         B, Hq, Hc, D, page_size, page_table.shape[1], page_table.shape[0],
         n_slots, max_context, split_tokens, scale, N.dtype_code(q.dtype), N.stream_ptr(q.device))
-    N.check(rc, "fp_paged_decode")
+    N.check(rc, entry)
     return out, lse
 
 

@@ -167,6 +167,44 @@ int fp_paged_decode(const void* q, int64_t q_stride_b, int64_t q_stride_h,
                     void* stream);
 
 /*
+ * The two passes of fp_paged_decode as separate calls, same arguments: the partial pass
+ * leaves, per (sequence, query head, split), the unnormalised accumulator, running
+ * maximum and denominator in the workspace ([B, Hq, n_splits, D] floats followed by
+ * [B, Hq, n_splits, 2] floats, log2 units); the merge pass combines them into out and
+ * lse.  For callers that time or overlap the passes, or that combine partials of one
+ * sequence held on several devices with the same merge.  No counterpart in the
+ * reference, whose Triton decode kernel keeps both passes internal
+ * (torch/_inductor/kernel/flex/flex_decoding.py:229).  When one split covers
+ * max_context the partial pass writes out and lse itself and the merge pass does nothing.
+ */
+int fp_paged_decode_partial(const void* q, int64_t q_stride_b, int64_t q_stride_h,
+                            const void* pool_k, const void* pool_v,
+                            const int64_t* page_table, int64_t pt_row_stride,
+                            const int64_t* batch_idx,
+                            const void* input_pos, int pos_index_type,
+                            void* out, int64_t out_stride_b, int64_t out_stride_h,
+                            float* lse,
+                            void* workspace, int64_t workspace_bytes,
+                            int32_t B, int32_t Hq, int32_t Hc, int32_t D,
+                            int32_t page_size, int32_t n_pages, int32_t max_batch,
+                            int64_t n_slots, int32_t max_context, int32_t split_tokens,
+                            float scale, int dtype,
+                            void* stream);
+int fp_paged_decode_merge(const void* q, int64_t q_stride_b, int64_t q_stride_h,
+                          const void* pool_k, const void* pool_v,
+                          const int64_t* page_table, int64_t pt_row_stride,
+                          const int64_t* batch_idx,
+                          const void* input_pos, int pos_index_type,
+                          void* out, int64_t out_stride_b, int64_t out_stride_h,
+                          float* lse,
+                          void* workspace, int64_t workspace_bytes,
+                          int32_t B, int32_t Hq, int32_t Hc, int32_t D,
+                          int32_t page_size, int32_t n_pages, int32_t max_batch,
+                          int64_t n_slots, int32_t max_context, int32_t split_tokens,
+                          float scale, int dtype,
+                          void* stream);
+
+/*
  * Per-row key limits of the hybrid mask (bidirectional inside an image span,
  * causal elsewhere).  Replaces the compiled create_block_mask evaluation of
  * create_prefill_blockmask (paged_attention.py:343-362) with

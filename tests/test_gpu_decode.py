@@ -199,3 +199,21 @@ def test_attention_callable_with_engine_masks():
         torch.cuda.synchronize()
         e_out, e_aux = A.compiled_flex_attn_decode(static_q, K, V, block_mask=mask, return_aux=AuxRequest(lse=True))
         assert torch.equal(g_out, e_out) and torch.equal(g_aux.lse, e_aux.lse)
+
+
+def test_partial_then_merge_equals_the_fused_call():
+    dtype = torch.bfloat16
+    st = PagedState(7, n_pages=96, page_size=32, max_batch=6, Hc=2, D=128, dtype=dtype)
+    for L in (700, 64, 1300):
+        st.add_sequence(L)
+    st.prefill_random()
+    q = randn(st.gen, (3, 4, 1, 128), dtype)
+    pos = torch.tensor([699, 63, 1299], dtype=torch.int32)
+    ws = torch.zeros(ops.decode_workspace_bytes(3, 4, 128, 1408, 256), dtype=torch.uint8, device=DEV)
+    both = run_decode(st, q, pos, split_tokens=256, max_context=1408, workspace=ws)
+    out = torch.zeros_like(both[0])
+    lse = torch.zeros_like(both[1])
+    run_decode(st, q, pos, split_tokens=256, max_context=1408, workspace=ws, out=out, lse=lse, phase="partial")
+    assert not out.any()  # the partial pass leaves out untouched when there are several splits
+    run_decode(st, q, pos, split_tokens=256, max_context=1408, workspace=ws, out=out, lse=lse, phase="merge")
+    assert torch.equal(out, both[0]) and torch.equal(lse, both[1])
