@@ -45,7 +45,7 @@ DTYPES = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
 
 # HBM bytes per launch of paged_decode_kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # (profiles/), scaled by the same counters on a plain copy of known size; None = not measured
-TRAFFIC_BYTES = {}
+TRAFFIC_BYTES = {"cfg2": 671.7e6}  # profiles/paged_decode_cfg2_hbm_traffic.md
 
 
 @dataclass
@@ -428,7 +428,7 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--decode-only", action="store_true", help="skip the append/gather/prefill side measurements")
     ap.add_argument("--pmc-calibration", action="store_true",
-                    help="also run a plain 1 GiB device copy a few times, so a rocprofv3 --pmc run of this "
+                    help="also run a plain 1 GiB elementwise copy (x * 2) a few times, so a rocprofv3 --pmc run of this "
                          "command holds a kernel of known traffic next to the decode kernel")
     ap.add_argument("--hbm-budget-gb", type=float, default=None, help="pool size for cfg5")
     args = ap.parse_args()
@@ -451,7 +451,7 @@ def main() -> int:
         src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")  # 1 GiB read + 1 GiB written per copy
         dst = torch.empty_like(src)
         for _ in range(5):
-            dst.copy_(src)
+            torch.mul(src, 2.0, out=dst)  # an elementwise kernel of its own name: reads 1 GiB, writes 1 GiB
         torch.cuda.synchronize()
         del src, dst
 
