@@ -68,6 +68,11 @@ struct BF16 {
   static __device__ __forceinline__ short from_float(float x) {
     return __builtin_bit_cast(short, static_cast<__bf16>(x));
   }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    const bf16x2 v = {static_cast<__bf16>(lo), static_cast<__bf16>(hi)};
+    return __builtin_bit_cast(uint32_t, v);
+  }
 };
 struct F16 {
   using vec8 = f16x8;
@@ -77,7 +82,14 @@ struct F16 {
   static __device__ __forceinline__ short from_float(float x) {
     return __builtin_bit_cast(short, static_cast<_Float16>(x));
   }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+    const f16x2 v = {static_cast<_Float16>(lo), static_cast<_Float16>(hi)};
+    return __builtin_bit_cast(uint32_t, v);
+  }
 };
+
+constexpr f32x16 kZero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
@@ -87,8 +99,8 @@ __device__ __forceinline__ s16x4 lds_read_tr(const char* p) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(p));
 }
 
-template <typename E, int D, int MB>
-__global__ __launch_bounds__(kThreads) void paged_prefill_kernel(const PrefillArgs a) {
+template <typename E, int D, int MB, bool kPow2>
+__global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const PrefillArgs a) {
   constexpr int BM = kWaves * 32 * MB;     // query rows per workgroup
   constexpr int RS = D * 2 + 16;           // LDS row stride in bytes (16-byte pad: no bank conflicts)
   constexpr int CPR = D * 2 / 16;          // 16-byte chunks per K/V row
@@ -129,9 +141,11 @@ __global__ __launch_bounds__(kThreads) void paged_prefill_kernel(const PrefillAr
 
   int run0 = 0;
   while (run0 < BM) {
-    const int sq = s_bidx[run0];
+    // values every lane agrees on are moved to scalar registers so the control flow that
+    // depends on them stays uniform
+    const int sq = __builtin_amdgcn_readfirstlane(s_bidx[run0]);
     int run1 = run0 + 1;
-    while (run1 < BM && s_bidx[run1] == sq) ++run1;
+    while (run1 < BM && __builtin_amdgcn_readfirstlane(s_bidx[run1]) == sq) ++run1;
 
     // rows of this wavefront: block mb covers tile rows wave*32*MB + mb*32 + ln
     int row[MB], lim[MB];
@@ -166,18 +180,21 @@ __global__ __launch_bounds__(kThreads) void paged_prefill_kernel(const PrefillAr
     int wave_max = my_max;
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) wave_max = max(wave_max, __shfl_xor(wave_max, off));
+    wave_max = __builtin_amdgcn_readfirstlane(wave_max);
     int wave_min = 0x7fffffff;  // smallest limit among the active rows (tiles below it need no masking)
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
       if (active[mb]) wave_min = min(wave_min, lim[mb]);
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) wave_min = min(wave_min, __shfl_xor(wave_min, off));
+    wave_min = __builtin_amdgcn_readfirstlane(wave_min);
     __syncthreads();  // s_red and the LDS tiles of the previous run are free
     if (lane == 0) s_red[wave] = wave_max;
     __syncthreads();
     int kv_max = 0;
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) kv_max = max(kv_max, s_red[w]);
+    kv_max = __builtin_amdgcn_readfirstlane(kv_max);
     const int n_kv_tiles = (kv_max + kTileN - 1) / kTileN;
 
     // Q^T operands: lane (query ln, half) holds d = 16*ds + 8*half .. +8 for every k-step
@@ -200,43 +217,44 @@ __global__ __launch_bounds__(kThreads) void paged_prefill_kernel(const PrefillAr
       m_run[mb] = -INFINITY;
       l_run[mb] = 0.f;
 #pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) o_acc[mb][db][i] = 0.f;
+      for (int db = 0; db < DB; ++db) o_acc[mb][db] = kZero16;
     }
 
     // ---- K/V fetch pipeline: page ids two tiles ahead, rows one tile ahead ----
     const int64_t* pt_row = a.page_table + static_cast<int64_t>(sq) * a.pt_row_stride;
-    int64_t slot_next[NI];  // pool slot of this thread's rows in the tile about to be fetched
+    // pool slot of this thread's rows in the tile about to be fetched; -1 = no such key.
+    // Lookups and loads are branch-free: an absent row reads slot 0 and is zeroed afterwards.
+    int slot_next[NI];
     v4u kst[NI], vst[NI];
+    bool fetched[NI];  // whether the row held in kst/vst exists
 
-    auto lookup = [&](int kt, int64_t (&slot)[NI]) {
+    auto lookup = [&](int kt, int (&slot)[NI]) {
 #pragma unroll
       for (int i = 0; i < NI; ++i) {
         const int c = tid + i * kThreads;
         const int kpos = kt * kTileN + c / CPR;
-        slot[i] = -1;
-        if (kpos < kv_max) {
-          int64_t blk;
-          int off;
-          a.pd.split(kpos, blk, off);
-          if (blk < a.n_pages) {
-            const int64_t page = pt_row[blk];
-            if (page >= 0 && page < a.n_pages) slot[i] = page * a.pd.page_size + off;
-          }
+        int blk, off;
+        if (kPow2) {  // page size is a power of two: shift and mask, no branch on the page size
+          blk = kpos >> a.pd.shift;
+          off = kpos & (a.pd.page_size - 1);
+        } else {
+          blk = kpos / a.pd.page_size;
+          off = kpos - blk * a.pd.page_size;
         }
+        const bool in_range = kpos < kv_max && blk < a.n_pages;
+        const int64_t page = pt_row[in_range ? blk : 0];
+        const bool ok = in_range && page >= 0 && page < a.n_pages;
+        slot[i] = ok ? static_cast<int>(page) * a.pd.page_size + off : -1;
       }
     };
-    auto fetch = [&](const int64_t (&slot)[NI]) {
+    auto fetch = [&](const int (&slot)[NI]) {
 #pragma unroll
       for (int i = 0; i < NI; ++i) {
         const int cc = (tid + i * kThreads) % CPR;
-        kst[i] = v4u{0, 0, 0, 0};
-        vst[i] = v4u{0, 0, 0, 0};
-        if (slot[i] >= 0) {
-          kst[i] = *reinterpret_cast<const v4u*>(kplane + slot[i] * (D * 2) + cc * 16);
-          vst[i] = *reinterpret_cast<const v4u*>(vplane + slot[i] * (D * 2) + cc * 16);
-        }
+        fetched[i] = slot[i] >= 0;
+        const int64_t byte = (static_cast<int64_t>(fetched[i] ? slot[i] : 0) * (D * 2)) + cc * 16;
+        kst[i] = *reinterpret_cast<const v4u*>(kplane + byte);
+        vst[i] = *reinterpret_cast<const v4u*>(vplane + byte);
       }
     };
     auto stage = [&](int buf) {
@@ -244,8 +262,8 @@ __global__ __launch_bounds__(kThreads) void paged_prefill_kernel(const PrefillAr
       for (int i = 0; i < NI; ++i) {
         const int c = tid + i * kThreads;
         const int off = (c / CPR) * RS + (c % CPR) * 16;
-        *reinterpret_cast<v4u*>(&s_k[buf][off]) = kst[i];
-        *reinterpret_cast<v4u*>(&s_v[buf][off]) = vst[i];
+        *reinterpret_cast<v4u*>(&s_k[buf][off]) = fetched[i] ? kst[i] : v4u{0, 0, 0, 0};
+        *reinterpret_cast<v4u*>(&s_v[buf][off]) = fetched[i] ? vst[i] : v4u{0, 0, 0, 0};
       }
     };
 
@@ -261,7 +279,7 @@ __global__ __launch_bounds__(kThreads) void paged_prefill_kernel(const PrefillAr
       const int buf = kt & 1;
       const bool more = kt + 1 < n_kv_tiles;
       if (more) fetch(slot_next);          // rows of tile kt+1 (their slots were looked up a tile ago)
-      int64_t slot_after[NI];
+      int slot_after[NI];
       if (more) lookup(kt + 2, slot_after);
 
       const int key0 = kt * kTileN;
@@ -271,9 +289,7 @@ __global__ __launch_bounds__(kThreads) void paged_prefill_kernel(const PrefillAr
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-          for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) s_acc[mb][kb][i] = 0.f;
+          for (int kb = 0; kb < 2; ++kb) s_acc[mb][kb] = kZero16;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
@@ -286,45 +302,51 @@ __global__ __launch_bounds__(kThreads) void paged_prefill_kernel(const PrefillAr
         }
 
         // ---- online softmax, one query per lane ----
+        // Scores are handled as plain scalars (element writes into the MFMA vector types
+        // make the compiler copy whole vectors), P is packed two values per register.
         const bool need_mask = key0 + kTileN > wave_min;
         s16x8 p_op[MB][4];  // P^T as B operands of the 4 k-steps (16 keys each)
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
-          float mx = -INFINITY;
+          float sc[32];
 #pragma unroll
-          for (int kb = 0; kb < 2; ++kb) {
+          for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-              float sv = s_acc[mb][kb][i];
-              if (need_mask) {
-                const int key = key0 + kb * 32 + (i >> 2) * 8 + half * 4 + (i & 3);
-                sv = key < lim[mb] ? sv : -INFINITY;
-                s_acc[mb][kb][i] = sv;
-              }
-              mx = fmaxf(mx, sv);
+            for (int i = 0; i < 16; ++i) sc[kb * 16 + i] = s_acc[mb][kb][i];
+          if (need_mask) {
+            // register i of block kb is key kb*32 + (i/4)*8 + half*4 + i%4 of the tile
+            const int rel = lim[mb] - key0 - half * 4;
+#pragma unroll
+            for (int x = 0; x < 32; ++x) {
+              const int key = (x >> 4) * 32 + ((x & 15) >> 2) * 8 + (x & 3);
+              sc[x] = key < rel ? sc[x] : -INFINITY;
             }
           }
+          float mx = sc[0];
+#pragma unroll
+          for (int x = 1; x < 32; ++x) mx = fmaxf(mx, sc[x]);
           mx = fmaxf(mx, __shfl_xor(mx, 32));
           const float m_new = fmaxf(m_run[mb], mx * a.qscale);
           const float m_safe = m_new == -INFINITY ? 0.f : m_new;
           const float alpha = fast_exp2(m_run[mb] - m_safe);
           m_run[mb] = m_new;
           float psum = 0.f;
+          uint32_t pw[16];
 #pragma unroll
-          for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-              const float p = fast_exp2(fmaf(s_acc[mb][kb][i], a.qscale, -m_safe));
-              psum += p;
-              p_op[mb][kb * 2 + (i >> 3)][i & 7] = E::from_float(p);
-            }
+          for (int x = 0; x < 32; x += 2) {
+            const float p0 = fast_exp2(fmaf(sc[x], a.qscale, -m_safe));
+            const float p1 = fast_exp2(fmaf(sc[x + 1], a.qscale, -m_safe));
+            psum += p0 + p1;
+            pw[x >> 1] = E::pack2(p0, p1);
           }
+          // k-step j takes registers 8j .. 8j+7 of the 32 scores = words 4j .. 4j+3
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            p_op[mb][j] = __builtin_bit_cast(s16x8, v4u{pw[4 * j], pw[4 * j + 1], pw[4 * j + 2], pw[4 * j + 3]});
           l_run[mb] = l_run[mb] * alpha + psum;
           if (__any(alpha != 1.f)) {
 #pragma unroll
-            for (int db = 0; db < DB; ++db)
-#pragma unroll
-              for (int i = 0; i < 16; ++i) o_acc[mb][db][i] *= alpha;
+            for (int db = 0; db < DB; ++db) o_acc[mb][db] *= alpha;
           }
         }
 
@@ -391,7 +413,10 @@ void launch(const PrefillArgs& a0, hipStream_t st) {
   a.n_tiles = (a.Lq + BM - 1) / BM;
   const int G = a.Hq / a.Hc;
   dim3 grid(a.Hc, G * a.n_tiles);
-  hipLaunchKernelGGL((paged_prefill_kernel<E, D, MB>), grid, dim3(kThreads), 0, st, a);
+  if (a.pd.shift >= 0)
+    hipLaunchKernelGGL((paged_prefill_kernel<E, D, MB, true>), grid, dim3(kThreads), 0, st, a);
+  else
+    hipLaunchKernelGGL((paged_prefill_kernel<E, D, MB, false>), grid, dim3(kThreads), 0, st, a);
 }
 
 }  // namespace
@@ -411,6 +436,7 @@ extern "C" int fp_paged_prefill(const void* q, int64_t q_stride_row, int64_t q_s
   if (n_slots < static_cast<int64_t>(n_pages) * page_size)
     return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_prefill: n_slots smaller than n_pages * page_size");
   if (Hc > 65535) return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill: Hc exceeds 65535");
+  if (n_slots > INT32_MAX) return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill: more than 2^31-1 slots per head");
   if (Lq == 0) return FP_OK;
   if (!q || !pool_k || !pool_v || !page_table || !batch_idx || !row_limit || !out || !lse)
     return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_prefill: null pointer");
