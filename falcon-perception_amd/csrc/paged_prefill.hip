@@ -15,8 +15,9 @@
 //         (plus one exchange between the two lane halves).
 //   O^T = V^T P^T: P^T is already in B-operand layout in the S^T accumulators; V^T
 //         comes out of LDS through ds_read_b64_tr_b16, so V is staged row-major like K.
-//   K/V tiles of 64 keys are fetched page by page with 16-byte loads one tile ahead
-//   (registers), page ids two tiles ahead, and double-buffered in LDS.
+//   K/V tiles of 64 keys are fetched page by page one tile ahead with global_load_lds
+//   (16 bytes per lane straight into LDS, no staging registers), page ids two tiles ahead,
+//   into a double buffer whose rows are chunk-permuted against bank conflicts.
 // Rows of one 128-row tile may belong to several sequences: the tile is processed one
 // run of equal batch_idx at a time; rows of slot 0 are padding (out 0, lse -inf).
 #include "fp_common.h"
@@ -30,6 +31,7 @@ namespace {
 constexpr int kWaves = 4;
 constexpr int kThreads = kWaves * 64;
 constexpr int kTileN = 64;  // keys per tile
+constexpr int kPrefetch = 3; // LDS operand reads in flight ahead of the MFMA that uses them
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
@@ -99,18 +101,45 @@ __device__ __forceinline__ s16x4 lds_read_tr(const char* p) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(p));
 }
 
+template <int N>
+struct IntC {
+  static constexpr int value = N;
+};
+
+// K/V tiles in LDS are 64 unpadded rows of D * 2 bytes, filled by global_load_lds (each lane's
+// 16 bytes land at base + lane * 16).  Bank conflicts are avoided by permuting the 16-byte chunks
+// of a row on the GLOBAL side of the load:
+//   K: chunk c of row r sits at position c ^ kswz(r).  The MFMA operand read takes the same chunk
+//      of 16 consecutive rows, which then fall into 16 different positions.
+//   V: the 32-byte region c32 of row r sits at region (c32 + vrot(r)) mod regions.  The transpose
+//      read takes 4 consecutive rows x 32 bytes per 16-lane block, two blocks side by side.
+template <int D>
+struct Swizzle {
+  static constexpr int CPR = D * 2 / 16;  // 16-byte chunks per row
+  static constexpr int R32 = CPR / 2;     // 32-byte regions per row
+  static __device__ __forceinline__ int kswz(int r) { return (r / (16 / CPR)) % CPR; }
+  static __device__ __forceinline__ int vrot(int r) { return (2 * ((r / (8 / R32)) & 3)) % R32; }
+};
+
 template <typename E, int D, int MB, bool kPow2>
 __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const PrefillArgs a) {
+  using SW = Swizzle<D>;
   constexpr int BM = kWaves * 32 * MB;     // query rows per workgroup
-  constexpr int RS = D * 2 + 16;           // LDS row stride in bytes (16-byte pad: no bank conflicts)
-  constexpr int CPR = D * 2 / 16;          // 16-byte chunks per K/V row
-  constexpr int NI = kTileN * CPR / kThreads;  // chunks per thread per tile and tensor
+  constexpr int ROWB = D * 2;              // bytes of a K/V row
+  constexpr int CPR = SW::CPR;
+  constexpr int R32 = SW::R32;
+  constexpr int RPI = 64 / CPR;            // rows one wavefront load instruction brings in
+  constexpr int NI = kTileN / (RPI * kWaves);  // load instructions per wavefront, tile and tensor
   constexpr int DS = D / 16;               // MFMA k-steps over head_dim
   constexpr int DB = D / 32;               // 32-wide blocks of head_dim in O^T
-  constexpr int TILE_BYTES = kTileN * RS;
+  constexpr int TILE_BYTES = kTileN * ROWB;
 
-  __shared__ __attribute__((aligned(16))) char s_k[2][TILE_BYTES];
-  __shared__ __attribute__((aligned(16))) char s_v[2][TILE_BYTES];
+  // four separate arrays (not one indexed array) so that a load into one buffer is known not to
+  // alias the reads of the other
+  __shared__ __attribute__((aligned(1024))) char s_k0[TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) char s_k1[TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) char s_v0[TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) char s_v1[TILE_BYTES];
   __shared__ int s_bidx[BM];
   __shared__ int s_red[kWaves];
 
@@ -126,18 +155,33 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
   const int lane = tid & 63;
   const int half = lane >> 5;   // which 8 of 16 k-values / which 4 of 8 rows this lane holds
   const int ln = lane & 31;     // query column (S^T, O^T) or key row (K operand)
+  const int blk = lane >> 4;    // 16-lane block of the transpose read
+  const int bi = lane & 15;
   const int tile0 = tile * BM;
 
   for (int i = tid; i < BM; i += kThreads) {
     const int r = tile0 + i;
-    int64_t bi = r < a.Lq ? a.batch_idx[r] : 0;
-    if (bi < 0 || bi >= a.max_batch) bi = 0;
-    s_bidx[i] = static_cast<int>(bi);
+    int64_t bx = r < a.Lq ? a.batch_idx[r] : 0;
+    if (bx < 0 || bx >= a.max_batch) bx = 0;
+    s_bidx[i] = static_cast<int>(bx);
   }
   __syncthreads();
 
-  const char* kplane = a.pool_k + static_cast<int64_t>(hc) * a.n_slots * (D * 2);
-  const char* vplane = a.pool_v + static_cast<int64_t>(hc) * a.n_slots * (D * 2);
+  const char* kplane = a.pool_k + static_cast<int64_t>(hc) * a.n_slots * ROWB;
+  const char* vplane = a.pool_v + static_cast<int64_t>(hc) * a.n_slots * ROWB;
+
+  // ---- per-lane constants of the staging loads and of the operand reads ----
+  // load instruction i of this wavefront fills LDS rows (i * kWaves + wave) * RPI .. + RPI; this lane
+  // fills position lp of row lrow in that group.  kswz / vrot of the row do not depend on i.
+  const int lrow = lane / CPR;
+  const int lp = lane % CPR;
+  const int st_row0 = wave * RPI + lrow;  // row of load instruction 0; instruction i adds i * kWaves * RPI
+  const int k_src_off = (lp ^ SW::kswz(st_row0)) * 16;
+  const int v_src_off = ((((lp >> 1) + R32 - SW::vrot(st_row0)) % R32) * 2 + (lp & 1)) * 16;
+  // K operand: row kb * 32 + ln, chunk 2 * ds + half at position (2 * ds) ^ ksel
+  const int ksel = half ^ SW::kswz(ln);
+  // V operand: rows keyb .. , region (2 * db + vsel) % R32, 8 bytes (bi & 3) inside it
+  const int vsel = (blk & 1) + SW::vrot(half * 4 + (bi >> 2));
 
   int run0 = 0;
   while (run0 < BM) {
@@ -220,67 +264,69 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
       for (int db = 0; db < DB; ++db) o_acc[mb][db] = kZero16;
     }
 
-    // ---- K/V fetch pipeline: page ids two tiles ahead, rows one tile ahead ----
+    // ---- K/V fetch pipeline: page ids two tiles ahead, rows one tile ahead straight into LDS ----
     const int64_t* pt_row = a.page_table + static_cast<int64_t>(sq) * a.pt_row_stride;
-    // pool slot of this thread's rows in the tile about to be fetched; -1 = no such key.
-    // Lookups and loads are branch-free: an absent row reads slot 0 and is zeroed afterwards.
-    int slot_next[NI];
-    v4u kst[NI], vst[NI];
-    bool fetched[NI];  // whether the row held in kst/vst exists
+    // Page ids of the rows this lane fetches for the next tile, as loaded (not yet turned into
+    // slots: using them right after the load would make the wavefront wait for every load in
+    // flight, the row fetches included).  A key that does not exist (past the run's last key, or
+    // an unmapped page) reads slot 0: finite bytes, and every such key is masked.
+    int64_t page_next[NI];
 
-    auto lookup = [&](int kt, int (&slot)[NI]) {
-#pragma unroll
-      for (int i = 0; i < NI; ++i) {
-        const int c = tid + i * kThreads;
-        const int kpos = kt * kTileN + c / CPR;
-        int blk, off;
-        if (kPow2) {  // page size is a power of two: shift and mask, no branch on the page size
-          blk = kpos >> a.pd.shift;
-          off = kpos & (a.pd.page_size - 1);
-        } else {
-          blk = kpos / a.pd.page_size;
-          off = kpos - blk * a.pd.page_size;
-        }
-        const bool in_range = kpos < kv_max && blk < a.n_pages;
-        const int64_t page = pt_row[in_range ? blk : 0];
-        const bool ok = in_range && page >= 0 && page < a.n_pages;
-        slot[i] = ok ? static_cast<int>(page) * a.pd.page_size + off : -1;
+    auto key_block = [&](int kpos, int& blkid, int& off) {
+      if (kPow2) {  // page size is a power of two: shift and mask, no branch on the page size
+        blkid = kpos >> a.pd.shift;
+        off = kpos & (a.pd.page_size - 1);
+      } else {
+        blkid = kpos / a.pd.page_size;
+        off = kpos - blkid * a.pd.page_size;
       }
     };
-    auto fetch = [&](const int (&slot)[NI]) {
+    auto lookup = [&](int kt, int64_t (&page)[NI]) {
 #pragma unroll
       for (int i = 0; i < NI; ++i) {
-        const int cc = (tid + i * kThreads) % CPR;
-        fetched[i] = slot[i] >= 0;
-        const int64_t byte = (static_cast<int64_t>(fetched[i] ? slot[i] : 0) * (D * 2)) + cc * 16;
-        kst[i] = *reinterpret_cast<const v4u*>(kplane + byte);
-        vst[i] = *reinterpret_cast<const v4u*>(vplane + byte);
+        const int kpos = kt * kTileN + i * kWaves * RPI + st_row0;
+        int blkid, off;
+        key_block(kpos, blkid, off);
+        page[i] = pt_row[(kpos < kv_max && blkid < a.n_pages) ? blkid : 0];
       }
     };
-    auto stage = [&](int buf) {
+    auto fetch = [&](int kt, const int64_t (&page)[NI], char* kdst, char* vdst) {
 #pragma unroll
       for (int i = 0; i < NI; ++i) {
-        const int c = tid + i * kThreads;
-        const int off = (c / CPR) * RS + (c % CPR) * 16;
-        *reinterpret_cast<v4u*>(&s_k[buf][off]) = fetched[i] ? kst[i] : v4u{0, 0, 0, 0};
-        *reinterpret_cast<v4u*>(&s_v[buf][off]) = fetched[i] ? vst[i] : v4u{0, 0, 0, 0};
+        const int kpos = kt * kTileN + i * kWaves * RPI + st_row0;
+        int blkid, off;
+        key_block(kpos, blkid, off);
+        const bool ok = kpos < kv_max && blkid < a.n_pages && page[i] >= 0 && page[i] < a.n_pages;
+        const int slot = ok ? static_cast<int>(page[i]) * a.pd.page_size + off : 0;
+        const int64_t rowbyte = static_cast<int64_t>(slot) * ROWB;
+        const int group = (i * kWaves + wave) * RPI * ROWB;  // wavefront-uniform LDS offset
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void*)(kplane + rowbyte + k_src_off),
+            (__attribute__((address_space(3))) void*)(kdst + group), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void*)(vplane + rowbyte + v_src_off),
+            (__attribute__((address_space(3))) void*)(vdst + group), 16, 0, 0);
       }
     };
 
     if (n_kv_tiles > 0) {
-      lookup(0, slot_next);
-      fetch(slot_next);
-      lookup(1, slot_next);
-      stage(0);
+      lookup(0, page_next);
+      fetch(0, page_next, s_k0, s_v0);
+      lookup(1, page_next);
     }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's rows have landed in LDS
     __syncthreads();
 
-    for (int kt = 0; kt < n_kv_tiles; ++kt) {
-      const int buf = kt & 1;
+    // one tile: start the fetch of the next tile into the other buffer, then work on this one
+    auto tile_step = [&](auto parity, int kt) {
+      constexpr int kBuf = decltype(parity)::value;
+      const char* kcur = kBuf ? s_k1 : s_k0;
+      const char* vcur = kBuf ? s_v1 : s_v0;
       const bool more = kt + 1 < n_kv_tiles;
-      if (more) fetch(slot_next);          // rows of tile kt+1 (their slots were looked up a tile ago)
-      int slot_after[NI];
-      if (more) lookup(kt + 2, slot_after);
+      if (more) {
+        fetch(kt + 1, page_next, kBuf ? s_k0 : s_k1, kBuf ? s_v0 : s_v1);
+        lookup(kt + 2, page_next);
+      }
 
       const int key0 = kt * kTileN;
       if (key0 < wave_max) {
@@ -290,14 +336,22 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
         for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
           for (int kb = 0; kb < 2; ++kb) s_acc[mb][kb] = kZero16;
+        // LDS operands are read kPrefetch steps ahead of the MFMA that consumes them
+        {
+          const char* krow = kcur + ln * ROWB;
+          auto read_k = [&](int t) {
+            const int kb = t / DS, ds = t % DS;
+            return *reinterpret_cast<const v4u*>(krow + kb * 32 * ROWB + (((2 * ds) ^ ksel) * 16));
+          };
+          v4u ring[kPrefetch];
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
+          for (int t = 0; t < kPrefetch; ++t) ring[t] = read_k(t);
 #pragma unroll
-          for (int ds = 0; ds < DS; ++ds) {
-            const v4u kw = *reinterpret_cast<const v4u*>(&s_k[buf][(kb * 32 + ln) * RS + (16 * ds + 8 * half) * 2]);
-            const s16x8 ka = __builtin_bit_cast(s16x8, kw);
+          for (int t = 0; t < 2 * DS; ++t) {
+            const s16x8 ka = __builtin_bit_cast(s16x8, ring[t % kPrefetch]);
+            if (t + kPrefetch < 2 * DS) ring[t % kPrefetch] = read_k(t + kPrefetch);
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb) s_acc[mb][kb] = E::mfma(ka, qreg[mb][ds], s_acc[mb][kb]);
+            for (int mb = 0; mb < MB; ++mb) s_acc[mb][t / DS] = E::mfma(ka, qreg[mb][t % DS], s_acc[mb][t / DS]);
           }
         }
 
@@ -351,32 +405,37 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
         }
 
         // ---- O^T += V^T P^T ----
-        const int blk = lane >> 4;   // 16-lane block of the transpose read
-        const int bi = lane & 15;
+        {
+          // step t = (j, db): this lane names the chunk (key = base + bi / 4, d = dblock + 4 * (bi % 4))
+          // and receives d = dblock + bi for keys base .. base + 3, once for each half of the 16 keys
+          const char* vrow = vcur + (half * 4 + (bi >> 2)) * ROWB + (bi & 3) * 8;
+          auto read_v = [&](int t, s16x4& lo, s16x4& hi) {
+            const int j = t / DB, db = t % DB;
+            const char* p0 = vrow + ((j >> 1) * 32 + (j & 1) * 16) * ROWB + ((2 * db + vsel) % R32) * 32;
+            lo = lds_read_tr(p0);
+            hi = lds_read_tr(p0 + 8 * ROWB);
+          };
+          s16x4 rlo[kPrefetch], rhi[kPrefetch];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+          for (int t = 0; t < kPrefetch; ++t) read_v(t, rlo[t], rhi[t]);
 #pragma unroll
-          for (int db = 0; db < DB; ++db) {
-            // this lane supplies the chunk (key = base + bi / 4, d = dblock + 4 * (bi % 4)) and receives
-            // d = dblock + bi for keys base .. base + 3
-            const int keyb = (j >> 1) * 32 + (j & 1) * 16 + half * 4 + (bi >> 2);
-            const int dcol = db * 32 + (blk & 1) * 16 + (bi & 3) * 4;
-            const char* p0 = &s_v[buf][keyb * RS + dcol * 2];
-            const s16x4 lo = lds_read_tr(p0);
-            const s16x4 hi = lds_read_tr(p0 + 8 * RS);
+          for (int t = 0; t < 4 * DB; ++t) {
+            const s16x4 lo = rlo[t % kPrefetch], hi = rhi[t % kPrefetch];
             const s16x8 va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            if (t + kPrefetch < 4 * DB) read_v(t + kPrefetch, rlo[t % kPrefetch], rhi[t % kPrefetch]);
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb) o_acc[mb][db] = E::mfma(va, p_op[mb][j], o_acc[mb][db]);
+            for (int mb = 0; mb < MB; ++mb) o_acc[mb][t % DB] = E::mfma(va, p_op[mb][t / DB], o_acc[mb][t % DB]);
           }
         }
       }
 
-      if (more) {
-        stage(buf ^ 1);
-#pragma unroll
-        for (int i = 0; i < NI; ++i) slot_next[i] = slot_after[i];
-      }
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // the rows fetched for the next tile have landed
       __syncthreads();
+    };
+
+    for (int kt = 0; kt < n_kv_tiles; kt += 2) {
+      tile_step(IntC<0>{}, kt);
+      if (kt + 1 < n_kv_tiles) tile_step(IntC<1>{}, kt + 1);
     }
 
     // ---- finish the run: normalise and store ----
@@ -392,10 +451,9 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
         for (int i4 = 0; i4 < 4; ++i4) {
           // registers 4*i4 .. 4*i4+3 hold d = db*32 + i4*8 + half*4 + 0..3
           const int d = db * 32 + i4 * 8 + half * 4;
-          s16x4 pk;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) pk[e] = E::from_float(o_acc[mb][db][i4 * 4 + e] * inv);
-          *reinterpret_cast<s16x4*>(o + d * 2) = pk;
+          const uint32_t w0 = E::pack2(o_acc[mb][db][i4 * 4 + 0] * inv, o_acc[mb][db][i4 * 4 + 1] * inv);
+          const uint32_t w1 = E::pack2(o_acc[mb][db][i4 * 4 + 2] * inv, o_acc[mb][db][i4 * 4 + 3] * inv);
+          *reinterpret_cast<uint2*>(o + d * 2) = uint2{w0, w1};
         }
       }
       if (half == 0)
