@@ -55,6 +55,10 @@ struct DecodeArgs {
   int split_tokens;
   int n_splits;
   float qscale;  // scale * log2(e)
+  // fused append (optional): the row of the newest token of every sequence, [B, Hc, 1, D]
+  const char* k_new;
+  const char* v_new;
+  int64_t kn_b, kn_h, vn_b, vn_h;  // bytes
 };
 
 // ---- element access: 16 bytes of a row -----------------------------------
@@ -269,6 +273,11 @@ __global__ __launch_bounds__(kThreads) void paged_decode_kernel(const DecodeArgs
     return;
   }
   const int t1 = static_cast<int>(L < t0 + a.split_tokens ? L : t0 + a.split_tokens);
+  // Fused append: the newest token (position L - 1) is not in the pool yet.  The workgroup whose
+  // range holds it reads that row from k_new / v_new, folds it in and writes it to its slot; the
+  // pool is only read up to L - 2.
+  const bool owns_new = a.k_new != nullptr && L - 1 >= t0;  // t1 == L whenever L - 1 lies in this split
+  const int t1_pool = (owns_new && t1 == L) ? t1 - 1 : t1;
 
   // page ids of this split -> LDS
   int64_t blk0;
@@ -307,7 +316,7 @@ __global__ __launch_bounds__(kThreads) void paged_decode_kernel(const DecodeArgs
   __syncthreads();
 
 #pragma nounroll
-  for (int c0 = t0 + wave * CH; c0 < t1; c0 += kWaves * CH) {
+  for (int c0 = t0 + wave * CH; c0 < t1_pool; c0 += kWaves * CH) {
     v4u kreg[U], vreg[U];
     if (kAligned) {
       // the CH rows of this iteration lie in one page: one base, constant offsets
@@ -324,7 +333,7 @@ __global__ __launch_bounds__(kThreads) void paged_decode_kernel(const DecodeArgs
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         int t = c0 + u * RPW + grp;
-        if (t >= t1) t = t1 - 1;
+        if (t >= t1_pool) t = t1_pool - 1;
         int64_t blk;
         int off;
         a.pd.split(t, blk, off);
@@ -333,10 +342,31 @@ __global__ __launch_bounds__(kThreads) void paged_decode_kernel(const DecodeArgs
         vreg[u] = stream_load(vbase + slot * ROWB);
       }
     }
-    if (c0 + CH <= t1)
-      fold_rows<E, TPR, G, U, RPW, false>(kreg, vreg, q, a.qscale, c0 + grp, t1, m, l, acc);
+    if (c0 + CH <= t1_pool)
+      fold_rows<E, TPR, G, U, RPW, false>(kreg, vreg, q, a.qscale, c0 + grp, t1_pool, m, l, acc);
     else
-      fold_rows<E, TPR, G, U, RPW, true>(kreg, vreg, q, a.qscale, c0 + grp, t1, m, l, acc);
+      fold_rows<E, TPR, G, U, RPW, true>(kreg, vreg, q, a.qscale, c0 + grp, t1_pool, m, l, acc);
+  }
+
+  if (t1_pool != t1 && wave == 0) {
+    // the newest token: one row, held by lane group 0; every other row of this pass is masked
+    v4u kreg[U], vreg[U];
+    const v4u kn = *reinterpret_cast<const v4u*>(a.k_new + b * a.kn_b + hc * a.kn_h + col * 16);
+    const v4u vn = *reinterpret_cast<const v4u*>(a.v_new + b * a.vn_b + hc * a.vn_h + col * 16);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      kreg[u] = kn;
+      vreg[u] = vn;
+    }
+    fold_rows<E, TPR, G, U, RPW, true>(kreg, vreg, q, a.qscale, t1 - 1 + grp, t1, m, l, acc);
+    if (grp == 0) {
+      int64_t blk;
+      int off;
+      a.pd.split(t1 - 1, blk, off);
+      const int64_t slot = static_cast<int64_t>(s_pages[blk - blk0]) * a.pd.page_size + off;
+      __builtin_nontemporal_store(kn, reinterpret_cast<v4u*>(const_cast<char*>(kbase) + slot * ROWB));
+      __builtin_nontemporal_store(vn, reinterpret_cast<v4u*>(const_cast<char*>(vbase) + slot * ROWB));
+    }
   }
 
   // combine the lane groups of this wavefront
@@ -506,7 +536,13 @@ extern "C" int64_t fp_paged_decode_workspace_bytes(int32_t B, int32_t Hq, int32_
 
 namespace {
 
-int decode_entry(int phases, const void* q, int64_t q_stride_b, int64_t q_stride_h, const void* pool_k,
+struct NewRows {
+  const void* k;
+  const void* v;
+  int64_t k_stride_b, k_stride_h, v_stride_b, v_stride_h;  // elements
+};
+
+int decode_entry(int phases, const NewRows* fresh, const void* q, int64_t q_stride_b, int64_t q_stride_h, const void* pool_k,
                  const void* pool_v, const int64_t* page_table, int64_t pt_row_stride,
                  const int64_t* batch_idx, const void* input_pos, int pos_index_type,
                  void* out, int64_t out_stride_b, int64_t out_stride_h, float* lse,
@@ -549,7 +585,20 @@ int decode_entry(int phases, const void* q, int64_t q_stride_b, int64_t q_stride
                page_table, pt_row_stride, batch_idx, input_pos, pos_index_type == FP_INDEX_I64,
                static_cast<char*>(out), out_stride_b * eb, out_stride_h * eb, lse,
                nullptr, nullptr, Hq, Hc, fp::PageDiv(page_size), n_pages, max_batch, n_slots,
-               max_context, split_tokens, ns, scale * kLog2e};  // scores are kept in log2 units
+               max_context, split_tokens, ns, scale * kLog2e,  // scores are kept in log2 units
+               nullptr, nullptr, 0, 0, 0, 0};
+  if (fresh) {
+    if (!fresh->k || !fresh->v) return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode_append: null k_new / v_new");
+    if (!fp::aligned(fresh->k, 16) || !fp::aligned(fresh->v, 16) || (fresh->k_stride_b * eb) % 16 ||
+        (fresh->k_stride_h * eb) % 16 || (fresh->v_stride_b * eb) % 16 || (fresh->v_stride_h * eb) % 16)
+      return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode_append: k_new / v_new rows must be 16-byte aligned");
+    a.k_new = static_cast<const char*>(fresh->k);
+    a.v_new = static_cast<const char*>(fresh->v);
+    a.kn_b = fresh->k_stride_b * eb;
+    a.kn_h = fresh->k_stride_h * eb;
+    a.vn_b = fresh->v_stride_b * eb;
+    a.vn_h = fresh->v_stride_h * eb;
+  }
   if (ns > 1) {
     const int64_t need = static_cast<int64_t>(B) * Hq * ns * (D + 2) * static_cast<int64_t>(sizeof(float));
     if (!workspace || workspace_bytes < need || !fp::aligned(workspace, 16))
@@ -584,6 +633,13 @@ int decode_entry(int phases, const void* q, int64_t q_stride_b, int64_t q_stride
       pos_index_type, out, out_stride_b, out_stride_h, lse, workspace, workspace_bytes, B, Hq, Hc, D,     \
       page_size, n_pages, max_batch, n_slots, max_context, split_tokens, scale, dtype, stream
 
-extern "C" int fp_paged_decode(FP_DECODE_PARAMS) { return decode_entry(kPhasePartial | kPhaseMerge, FP_DECODE_ARGS); }
-extern "C" int fp_paged_decode_partial(FP_DECODE_PARAMS) { return decode_entry(kPhasePartial, FP_DECODE_ARGS); }
-extern "C" int fp_paged_decode_merge(FP_DECODE_PARAMS) { return decode_entry(kPhaseMerge, FP_DECODE_ARGS); }
+extern "C" int fp_paged_decode(FP_DECODE_PARAMS) {
+  return decode_entry(kPhasePartial | kPhaseMerge, nullptr, FP_DECODE_ARGS);
+}
+extern "C" int fp_paged_decode_partial(FP_DECODE_PARAMS) { return decode_entry(kPhasePartial, nullptr, FP_DECODE_ARGS); }
+extern "C" int fp_paged_decode_merge(FP_DECODE_PARAMS) { return decode_entry(kPhaseMerge, nullptr, FP_DECODE_ARGS); }
+extern "C" int fp_paged_decode_append(const void* k_new, const void* v_new, int64_t k_stride_b, int64_t k_stride_h,
+                                      int64_t v_stride_b, int64_t v_stride_h, FP_DECODE_PARAMS) {
+  const NewRows fresh{k_new, v_new, k_stride_b, k_stride_h, v_stride_b, v_stride_h};
+  return decode_entry(kPhasePartial | kPhaseMerge, &fresh, FP_DECODE_ARGS);
+}

@@ -104,8 +104,12 @@ def decode_workspace_bytes(B: int, Hq: int, D: int, max_context: int, split_toke
 def paged_decode(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor, batch_idx: Tensor,
                  input_pos: Tensor, page_size: int, max_context: int, *, scale: float | None = None,
                  split_tokens: int = 0, workspace: Tensor | None = None,
-                 out: Tensor | None = None, lse: Tensor | None = None, phase: str = "both") -> tuple[Tensor, Tensor]:
+                 out: Tensor | None = None, lse: Tensor | None = None, phase: str = "both",
+                 k_new: Tensor | None = None, v_new: Tensor | None = None) -> tuple[Tensor, Tensor]:
     """Single-query paged attention.  q [B, Hq, 1, D]; pools [Hc, N, D]; returns out [B, Hq, 1, D], lse [B, Hq, 1].
+
+    With `k_new`, `v_new` [B, Hc, 1, D] the call is the whole decode step: the rows are appended at
+    `input_pos` (as `kv_append` with clamp would) and attended over in the same launch.
 
     `phase` = "both" (default), "partial" (split-K pass only, results stay in `workspace`) or
     "merge" (cross-split merge of a previous partial pass with the same arguments)."""
@@ -133,7 +137,18 @@ def paged_decode(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor, 
     if out.stride(3) != 1 or not lse.is_contiguous() or lse.dtype != torch.float32:
         raise RuntimeError("out rows must be dense and lse contiguous float32")
     entry = {"both": "fp_paged_decode", "partial": "fp_paged_decode_partial", "merge": "fp_paged_decode_merge"}[phase]
+    fresh = ()
+    if k_new is not None or v_new is not None:
+        if phase != "both" or k_new is None or v_new is None:
+            raise RuntimeError("the fused append needs both k_new and v_new and runs both passes")
+        N.require_cuda(k_new, v_new)
+        if k_new.shape != (B, Hc, 1, D) or v_new.shape != (B, Hc, 1, D) or k_new.dtype != q.dtype or v_new.dtype != q.dtype:
+            raise RuntimeError("k_new / v_new must be [B, Hc, 1, D] of the q dtype")
+        k_new, v_new = _rows(k_new), _rows(v_new)
+        entry = "fp_paged_decode_append"
+        fresh = (k_new.data_ptr(), v_new.data_ptr(), k_new.stride(0), k_new.stride(1), v_new.stride(0), v_new.stride(1))
     rc = getattr(N.lib(), entry)(
+        *fresh,
         q.data_ptr(), q.stride(0), q.stride(1), pool_k.data_ptr(), pool_v.data_ptr(),
         page_table.data_ptr(), page_table.stride(0), batch_idx.data_ptr(),
         input_pos.data_ptr(), N.index_code(input_pos),

@@ -205,6 +205,34 @@ int fp_paged_decode_merge(const void* q, int64_t q_stride_b, int64_t q_stride_h,
                           void* stream);
 
 /*
+ * Decode step in one call: append the newest K/V row of every sequence AND attend over the
+ * context including it.  Equivalent to fp_kv_append(clamp_negative = 1, S = 1) at position
+ * input_pos[b] followed by fp_paged_decode, i.e. to PagedKVCache.assign
+ * (paged_attention.py:184-232) + compiled_flex_attn_decode (model.py:150-162), without the
+ * separate append launch: the workgroup that owns position input_pos[b] takes that row from
+ * k_new / v_new, folds it into the attention and writes it to its pool slot.
+ *
+ *   k_new, v_new  [B, Hc, 1, D], element strides (b, h); pool_k / pool_v are written
+ * All other arguments as fp_paged_decode.
+ */
+int fp_paged_decode_append(const void* k_new, const void* v_new,
+                           int64_t k_stride_b, int64_t k_stride_h,
+                           int64_t v_stride_b, int64_t v_stride_h,
+                           const void* q, int64_t q_stride_b, int64_t q_stride_h,
+                           const void* pool_k, const void* pool_v,
+                           const int64_t* page_table, int64_t pt_row_stride,
+                           const int64_t* batch_idx,
+                           const void* input_pos, int pos_index_type,
+                           void* out, int64_t out_stride_b, int64_t out_stride_h,
+                           float* lse,
+                           void* workspace, int64_t workspace_bytes,
+                           int32_t B, int32_t Hq, int32_t Hc, int32_t D,
+                           int32_t page_size, int32_t n_pages, int32_t max_batch,
+                           int64_t n_slots, int32_t max_context, int32_t split_tokens,
+                           float scale, int dtype,
+                           void* stream);
+
+/*
  * Per-row key limits of the hybrid mask (bidirectional inside an image span,
  * causal elsewhere).  Replaces the compiled create_block_mask evaluation of
  * create_prefill_blockmask (paged_attention.py:343-362) with

@@ -217,3 +217,42 @@ def test_partial_then_merge_equals_the_fused_call():
     assert not out.any()  # the partial pass leaves out untouched when there are several splits
     run_decode(st, q, pos, split_tokens=256, max_context=1408, workspace=ws, out=out, lse=lse, phase="merge")
     assert torch.equal(out, both[0]) and torch.equal(lse, both[1])
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=str)
+@pytest.mark.parametrize("ctx", [320, 1280])
+def test_fused_append_decode_equals_append_then_decode(dtype, ctx):
+    """fp_paged_decode_append: same pool bits as the append kernel, same attention as the oracle.
+    Contexts include L = 1 (only the new token), split and page boundaries."""
+    P = 16
+    G = 2
+    outs = []
+    lens = [0, 1, P - 1, P, P + 1, 63, 64, 65, 127, 128, 300]  # tokens cached before the step
+    for fused in (False, True):
+        st = PagedState(8, n_pages=80, page_size=P, max_batch=13, Hc=2, D=128, dtype=dtype)
+        for L in lens:
+            st.add_sequence(L + 1)
+        st.lens = lens
+        st.prefill_random()
+        B = len(lens)
+        k1 = randn(st.gen, (B, 2, 1, 128), dtype)
+        v1 = randn(st.gen, (B, 2, 1, 128), dtype)
+        q = randn(st.gen, (B, 2 * G, 1, 128), dtype)
+        pos = torch.tensor(lens, dtype=torch.int32)
+        bidx = torch.tensor(st.slots, dtype=torch.int64, device=DEV)
+        pk, pv = st.pool_planes()
+        if fused:
+            out, lse = ops.paged_decode(q.to(DEV), pk, pv, st.cache.page_table, bidx, pos.to(DEV), P, ctx,
+                                        split_tokens=64, k_new=k1.to(DEV), v_new=v1.to(DEV))
+        else:
+            st.cache.insert_kv(0, k1.to(DEV), v1.to(DEV), input_pos=pos.view(B, 1).to(DEV), batch_idx=bidx)
+            out, lse = ops.paged_decode(q.to(DEV), pk, pv, st.cache.page_table, bidx, pos.to(DEV), P, ctx,
+                                        split_tokens=64)
+        outs.append((out, lse, st.cache.kv_cache.clone()))
+        if fused:
+            eo, el = oracle_decode(st, q, pos)
+            assert_close(out, lse, eo, el, dtype)
+    assert torch.equal(outs[0][2].view(torch.uint8), outs[1][2].view(torch.uint8))  # pools bit-identical
+    atol, rtol = TOL[dtype]
+    np.testing.assert_allclose(f64(outs[1][0]), f64(outs[0][0]), atol=atol, rtol=rtol)
+    np.testing.assert_allclose(f64(outs[1][1]), f64(outs[0][1]), atol=1e-4, rtol=1e-4)
