@@ -175,6 +175,15 @@ __device__ __forceinline__ void row_sum(float (&x)[kN]) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float safe_max(float m) { return m == -INFINITY ? 0.f : m; }
 
+// tokens per split of a context of L tokens: L is divided evenly over ceil(L / split_tokens)
+// splits, rounded up to 64 tokens (so every split starts on a wavefront-iteration boundary)
+__device__ __forceinline__ int split_part(int L, int split_tokens) {
+  if (L <= 0) return split_tokens;
+  const int n = (L + split_tokens - 1) / split_tokens;
+  const int even = (L + n - 1) / n;
+  return (even + 63) & ~63;
+}
+
 // One wavefront iteration: U row loads of K and V per lane are already in registers;
 // fold them into the lane group's online-softmax state.  kMasked: rows at or past
 // `t1` (only in the last iteration of a split) get a score of -inf.
@@ -260,7 +269,11 @@ __global__ __launch_bounds__(kThreads) void paged_decode_kernel(const DecodeArgs
   const int64_t trow = a.batch_idx[b];
   if (trow < 0 || trow >= a.max_batch) L = 0;
   if (L > a.max_context) L = a.max_context;
-  const int t0 = split * a.split_tokens;
+  // A context of L tokens is cut into ceil(L / split_tokens) parts of equal size (a multiple of
+  // 64 tokens), so the workgroups of one sequence carry the same load instead of leaving a short
+  // tail split.
+  const int part = split_part(static_cast<int>(L), a.split_tokens);
+  const int t0 = split * part;
   if (t0 >= L) {
     if (kDirect && split == 0) {
       // no visible key at all: out = 0, lse = -inf
@@ -272,7 +285,7 @@ __global__ __launch_bounds__(kThreads) void paged_decode_kernel(const DecodeArgs
     }
     return;
   }
-  const int t1 = static_cast<int>(L < t0 + a.split_tokens ? L : t0 + a.split_tokens);
+  const int t1 = static_cast<int>(L < t0 + part ? L : t0 + part);
   // Fused append: the newest token (position L - 1) is not in the pool yet.  The workgroup whose
   // range holds it reads that row from k_new / v_new, folds it in and writes it to its slot; the
   // pool is only read up to L - 2.
@@ -437,7 +450,8 @@ __global__ __launch_bounds__(64) void paged_decode_merge_kernel(const DecodeArgs
   const int64_t trow = a.batch_idx[b];
   if (trow < 0 || trow >= a.max_batch) L = 0;
   if (L > a.max_context) L = a.max_context;
-  const int ns = L <= 0 ? 0 : static_cast<int>((L + a.split_tokens - 1) / a.split_tokens);
+  const int part = split_part(static_cast<int>(L), a.split_tokens);
+  const int ns = L <= 0 ? 0 : static_cast<int>((L + part - 1) / part);
   const int64_t p0 = (static_cast<int64_t>(b) * a.Hq + hq) * a.n_splits;
 
   float mn = -INFINITY;
