@@ -518,8 +518,10 @@ int dispatch_dim(const DecodeArgs& a, int B, int D, int phases, hipStream_t st) 
   }
 }
 
+// Largest split (fewest partials to merge, least per-workgroup overhead) that still yields about
+// 2048 workgroups when every sequence is at max_context: 8 per CU to fill 256 CUs three deep.
 int default_split_tokens(int B, int Hc, int max_context, int page_size) {
-  int split = 1024;
+  int split = 2048;
   while (split > 128 && static_cast<int64_t>(B) * Hc * ((max_context + split - 1) / split) < 2048) split >>= 1;
   while (split / page_size + 2 > kMaxSplitPages) split >>= 1;
   return split < 64 ? 64 : split;

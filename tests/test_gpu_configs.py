@@ -1,0 +1,158 @@
+"""GPU: the larger BASELINE.json configurations as parity cases.
+
+cfg4  continuous-batching churn: mixed steps of 32 decode sequences and 4 prefill chunks of 1024
+      tokens, 25 % of the live pages freed and reused between steps, page size 64, GQA 2.
+cfg5  long-context decode on a pool sized to most of HBM (180 GB, shrunk to fit when the GPU
+      has less free memory): batch 256, 32 q / 8 kv heads, contexts 4096 + U[256, 12288].
+Full-size results are checked on sampled sequences / rows against the float64 oracle and through
+properties that do not depend on size.
+"""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from falcon_perception_amd import ops
+from falcon_perception_amd.paged_attention import PagedKVCache
+from oracle import paged_kv_oracle as O
+from tests.gpu_cases import DEV, f64
+
+pytestmark = pytest.mark.gpu
+
+ATOL, RTOL = 2e-2, 1e-2
+
+
+def gathered_oracle_decode(q, pool_k, pool_v, page_table, slot, ctx, P):
+    """Oracle for one sequence of a pool too large to copy to the host: gather the sequence on the
+    GPU (bit-exact, tested separately), attend densely in float64 on the CPU."""
+    dev = pool_k.device
+    lens = torch.tensor([ctx], device=dev)
+    slots = torch.tensor([slot], device=dev)
+    K = ops.kv_gather(pool_k, page_table, slots, lens, P, ctx)[0]
+    V = ops.kv_gather(pool_v, page_table, slots, lens, P, ctx)[0]
+    return O.masked_attention_dense(f64(q), f64(K), f64(V), np.ones((1, ctx), dtype=bool))
+
+
+def test_cfg4_continuous_batching_churn():
+    gen = torch.Generator().manual_seed(4)
+    dgen = torch.Generator(device=DEV).manual_seed(4)
+    P, Hq, Hc, D, n_pages = 64, 16, 8, 128, 8192
+    dtype = torch.bfloat16
+    cache = PagedKVCache(n_pages, P, 64, Hc, D, 1, dtype, device=DEV)
+    cache.free_pages = (torch.randperm(n_pages - 1, generator=gen) + 1).tolist()
+    cache.kv_cache.view(-1).normal_(generator=dgen)  # stale bytes everywhere, as after long service
+    pk, pv = cache.kv_cache[0, 0, 0], cache.kv_cache[0, 1, 0]
+    rnd = lambda *shape: torch.randn(shape, generator=dgen, device=DEV, dtype=torch.float32).to(dtype)
+
+    def admit(length):
+        b = cache.allocate()
+        cache.reserve(b, torch.tensor([b], device=DEV), length)
+        return b
+
+    def fill(slot, start, n):
+        """Append n random rows at positions start.. of a sequence (packed prefill append)."""
+        k, v = rnd(1, Hc, n, D), rnd(1, Hc, n, D)
+        bidx = torch.full((1, n), slot, dtype=torch.int64, device=DEV)
+        pos = torch.arange(start, start + n, dtype=torch.int64, device=DEV)[None]
+        cache.insert_kv(0, k, v, input_pos=pos, batch_idx=bidx)
+
+    ctx = {}
+    for L in torch.randint(512, 8193, (32,), generator=gen).tolist():
+        if not cache.can_reserve(L + 8):
+            break
+        s = admit(L + 8)
+        fill(s, 0, L)
+        ctx[s] = L
+    assert len(ctx) >= 24
+
+    for step in range(3):
+        # --- 4 prefill chunks of 1024 tokens: 2 fresh sequences whose first 512 tokens are an image
+        #     span, 2 sequences continuing after a 2048-token prefix already in pages
+        chunks = []
+        for kind in ("fresh", "fresh", "cont", "cont"):
+            if kind == "fresh":
+                s = admit(1024)
+                lim = [max(t + 1, 512) for t in range(1024)]
+                start = 0
+            else:
+                s = admit(2048 + 1024)
+                fill(s, 0, 2048)
+                lim = [2048 + t + 1 for t in range(1024)]
+                start = 2048
+            chunks.append((s, start, lim))
+        bidx = torch.cat([torch.full((1024,), s, dtype=torch.int64) for s, _, _ in chunks])[None].to(DEV)
+        pos = torch.cat([torch.arange(st, st + 1024, dtype=torch.int64) for _, st, _ in chunks])[None].to(DEV)
+        lim = torch.tensor([x for _, _, l in chunks for x in l], dtype=torch.int32, device=DEV)
+        k, v, q = rnd(1, Hc, 4096, D), rnd(1, Hc, 4096, D), rnd(1, Hq, 4096, D)
+        cache.insert_kv(0, k, v, input_pos=pos, batch_idx=bidx)
+        out, lse = ops.paged_prefill(q, pk, pv, cache.page_table, bidx, lim, P)
+        rows = np.arange(0, 4096, 61)  # sampled rows of every chunk
+        pt = cache.page_table.cpu().numpy()
+        eo, el = O.prefill_attention_paged(f64(q[:, :, rows]), pk.float().cpu().numpy(), pv.float().cpu().numpy(), pt,
+                                           bidx.cpu().numpy().reshape(-1)[rows], None, lim.cpu().numpy()[rows], P)
+        np.testing.assert_allclose(f64(out[:, :, rows]), eo, atol=ATOL, rtol=RTOL)
+        np.testing.assert_allclose(f64(lse[:, :, rows]), el, atol=2e-3, rtol=RTOL)
+
+        # --- decode step over every running sequence: fused append + attention
+        slots = sorted(ctx)
+        B = len(slots)
+        bt = torch.tensor(slots, dtype=torch.int64, device=DEV)
+        pt_ = torch.tensor([ctx[s] for s in slots], dtype=torch.int32, device=DEV)
+        k1, v1, q1 = rnd(B, Hc, 1, D), rnd(B, Hc, 1, D), rnd(B, Hq, 1, D)
+        o1, l1 = ops.paged_decode(q1, pk, pv, cache.page_table, bt, pt_, P, 8192 + 64, k_new=k1, v_new=v1)
+        for i in range(0, B, 5):
+            s = slots[i]
+            eo, el = gathered_oracle_decode(q1[i], pk, pv, cache.page_table, s, ctx[s] + 1, P)
+            np.testing.assert_allclose(f64(o1[i]), eo, atol=ATOL, rtol=RTOL)
+            np.testing.assert_allclose(f64(l1[i]), el, atol=2e-3, rtol=RTOL)
+            # the appended row is in its slot, bit for bit
+            page = cache.page_table_cpu[s][ctx[s] // P]
+            assert torch.equal(pk[:, page * P + ctx[s] % P].view(torch.int16), k1[i, :, 0].view(torch.int16))
+        for s in slots:
+            ctx[s] += 1
+
+        # --- churn: the chunk sequences leave, a quarter of the decode sequences are replaced
+        for s, _, _ in chunks:
+            cache.erase(s)
+        leaving = [slots[i] for i in torch.randperm(B, generator=gen)[: B // 4].tolist()]
+        for s in leaving:
+            cache.erase(s)
+            del ctx[s]
+        for L in torch.randint(512, 8193, (len(leaving),), generator=gen).tolist():
+            if cache.can_reserve(L + 8):
+                s = admit(L + 8)
+                fill(s, 0, L)
+                ctx[s] = L
+        live = [p for s in ctx for p in cache.page_table_cpu[s]]
+        assert len(live) == len(set(live)) and 0 not in live
+        assert len(live) + cache.num_free_pages == n_pages - 1
+
+
+def test_cfg5_long_context_decode_on_a_pool_sized_to_hbm():
+    import bench
+
+    free, total = torch.cuda.mem_get_info()
+    budget = min(180.0, (free - 24e9) / 1e9)
+    if budget < 30:
+        pytest.skip("not enough free HBM for a long-context pool")
+    case = bench.make_decode_case("cfg5", device=DEV, hbm_budget_gb=budget)
+    c = case.cfg
+    assert case.pool_k.numel() * 2 > 2**32  # byte offsets inside one plane need 64 bits
+    out, lse = case.run_fused()
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
+    # sampled sequences against the oracle: shortest, longest, and a few in between
+    order = np.argsort(case.lens)
+    for i in [order[0], order[-1], order[len(order) // 2], 0, c["B"] - 1]:
+        slot = int(case.batch_idx[i])
+        eo, el = gathered_oracle_decode(case.q[i], case.pool_k, case.pool_v, case.page_table, slot, case.lens[i] + 1,
+                                        case.page_size)
+        np.testing.assert_allclose(f64(out[i]), eo, atol=ATOL, rtol=RTOL)
+        np.testing.assert_allclose(f64(lse[i]), el, atol=2e-3, rtol=RTOL)
+    # split-count invariance on the whole batch
+    o2, l2 = ops.paged_decode(case.q, case.pool_k, case.pool_v, case.page_table, case.batch_idx, case.input_pos,
+                              case.page_size, case.max_context, split_tokens=512)
+    np.testing.assert_allclose(l2.cpu().numpy(), lse.cpu().numpy(), atol=1e-4, rtol=1e-5)
+    np.testing.assert_allclose(f64(o2), f64(out), atol=8e-3, rtol=8e-3)
