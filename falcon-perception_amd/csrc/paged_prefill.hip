@@ -8,8 +8,8 @@
 // arrives as one number per query row: keys 0..row_limit-1 of the row's own
 // sequence are visible.
 //
-// MFMA-bound.  A workgroup of 4 wavefronts owns kRowBlocks * 128 consecutive packed
-// query rows of one query head; a wavefront owns kRowBlocks blocks of 32 rows.
+// MFMA-bound.  A workgroup of 8 wavefronts owns one cache head and 256 / G consecutive packed
+// query rows of each of its G query heads; a wavefront owns 32 rows of one query head.
 //   S^T = K Q^T  (v_mfma_f32_32x32x16): keys are the M rows, queries the N columns, so a
 //         lane holds scores of ONE query and softmax row reductions stay in registers
 //         (plus one exchange between the two lane halves).
@@ -18,7 +18,7 @@
 //   K/V tiles of 64 keys are fetched page by page one tile ahead with global_load_lds
 //   (16 bytes per lane straight into LDS, no staging registers), page ids two tiles ahead,
 //   into a double buffer whose rows are chunk-permuted against bank conflicts.
-// Rows of one 128-row tile may belong to several sequences: the tile is processed one
+// Rows of one tile may belong to several sequences: the tile is processed one
 // run of equal batch_idx at a time; rows of slot 0 are padding (out 0, lse -inf).
 #include "fp_common.h"
 
@@ -28,9 +28,10 @@
 
 namespace {
 
-constexpr int kWaves = 4;
+constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * 64;
 constexpr int kTileN = 64;  // keys per tile
+constexpr float kMaxSlack = 6.f;  // the running maximum may lag a row's true maximum by this much (log2)
 constexpr int kPrefetch = 3; // LDS operand reads in flight ahead of the MFMA that uses them
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
@@ -121,10 +122,16 @@ struct Swizzle {
   static __device__ __forceinline__ int vrot(int r) { return (2 * ((r / (8 / R32)) & 3)) % R32; }
 };
 
-template <typename E, int D, int MB, bool kPow2>
+// G = query heads per cache head.  The 8 wavefronts of a workgroup are G heads x 8 / G blocks of
+// 32 query rows: every head of the group works from the same staged K/V tile, so the bytes that
+// travel from L2 into LDS (64 B per cycle and CU, and a wavefront waits at its load instructions
+// while that path is busy) are shared by all of them.
+template <typename E, int D, int G, bool kPow2>
 __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const PrefillArgs a) {
   using SW = Swizzle<D>;
-  constexpr int BM = kWaves * 32 * MB;     // query rows per workgroup
+  constexpr int MB = 1;                    // 32-row blocks per wavefront
+  constexpr int RB = kWaves / G;           // 32-row blocks per workgroup
+  constexpr int BM = RB * 32;              // query rows per workgroup
   constexpr int ROWB = D * 2;              // bytes of a K/V row
   constexpr int CPR = SW::CPR;
   constexpr int R32 = SW::R32;
@@ -143,15 +150,14 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
   __shared__ int s_bidx[BM];
   __shared__ int s_red[kWaves];
 
-  // linear id = cache head + Hc * (head in group + G * tile): all query heads and tiles that
-  // read one cache head run on the XCD that already holds its K/V in L2
-  const int G = a.Hq / a.Hc;
+  // linear id = cache head + Hc * tile: all tiles that read one cache head run on the XCD that
+  // already holds its K/V in L2
   const int hc = blockIdx.x;
-  const int g = blockIdx.y % G;
-  const int tile = a.n_tiles - 1 - blockIdx.y / G;  // longest key ranges first
-  const int hq = hc * G + g;
+  const int tile = a.n_tiles - 1 - blockIdx.y;  // longest key ranges first
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int hq = hc * G + wave % G;  // query head of this wavefront
+  const int rblock = wave / G;       // its block of 32 rows inside the tile
   const int lane = tid & 63;
   const int half = lane >> 5;   // which 8 of 16 k-values / which 4 of 8 rows this lane holds
   const int ln = lane & 31;     // query column (S^T, O^T) or key row (K operand)
@@ -191,13 +197,13 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
     int run1 = run0 + 1;
     while (run1 < BM && __builtin_amdgcn_readfirstlane(s_bidx[run1]) == sq) ++run1;
 
-    // rows of this wavefront: block mb covers tile rows wave*32*MB + mb*32 + ln
+    // rows of this wavefront: tile rows rblock * 32 + ln
     int row[MB], lim[MB];
     bool active[MB];
     int my_max = 0;
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
-      const int tr = wave * 32 * MB + mb * 32 + ln;
+      const int tr = (rblock * MB + mb) * 32 + ln;
       row[mb] = tile0 + tr;
       active[mb] = tr >= run0 && tr < run1 && row[mb] < a.Lq;
       lim[mb] = (active[mb] && sq != 0) ? a.row_limit[row[mb]] : 0;
@@ -290,23 +296,31 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
         page[i] = pt_row[(kpos < kv_max && blkid < a.n_pages) ? blkid : 0];
       }
     };
-    auto fetch = [&](int kt, const int64_t (&page)[NI], char* kdst, char* vdst) {
-#pragma unroll
-      for (int i = 0; i < NI; ++i) {
-        const int kpos = kt * kTileN + i * kWaves * RPI + st_row0;
-        int blkid, off;
-        key_block(kpos, blkid, off);
-        const bool ok = kpos < kv_max && blkid < a.n_pages && page[i] >= 0 && page[i] < a.n_pages;
-        const int slot = ok ? static_cast<int>(page[i]) * a.pd.page_size + off : 0;
-        const int64_t rowbyte = static_cast<int64_t>(slot) * ROWB;
-        const int group = (i * kWaves + wave) * RPI * ROWB;  // wavefront-uniform LDS offset
+    // One staging load: piece 2 * i is the K load of row group i, piece 2 * i + 1 its V load.
+    // The pieces of the next tile are issued one at a time between the MFMAs of the current
+    // tile: the CU moves 64 bytes per cycle from L2 towards LDS, and a burst of all pieces
+    // from all wavefronts at once would hold each wavefront at its load instructions.
+    auto fetch_piece = [&](int kt, int piece, const int64_t (&page)[NI], char* kdst, char* vdst) {
+      const int i = piece >> 1;
+      const int kpos = kt * kTileN + i * kWaves * RPI + st_row0;
+      int blkid, off;
+      key_block(kpos, blkid, off);
+      const bool ok = kpos < kv_max && blkid < a.n_pages && page[i] >= 0 && page[i] < a.n_pages;
+      const int slot = ok ? static_cast<int>(page[i]) * a.pd.page_size + off : 0;
+      const int64_t rowbyte = static_cast<int64_t>(slot) * ROWB;
+      const int group = (i * kWaves + wave) * RPI * ROWB;  // wavefront-uniform LDS offset
+      if ((piece & 1) == 0)
         __builtin_amdgcn_global_load_lds(
             (const __attribute__((address_space(1))) void*)(kplane + rowbyte + k_src_off),
             (__attribute__((address_space(3))) void*)(kdst + group), 16, 0, 0);
+      else
         __builtin_amdgcn_global_load_lds(
             (const __attribute__((address_space(1))) void*)(vplane + rowbyte + v_src_off),
             (__attribute__((address_space(3))) void*)(vdst + group), 16, 0, 0);
-      }
+    };
+    auto fetch = [&](int kt, const int64_t (&page)[NI], char* kdst, char* vdst) {
+#pragma unroll
+      for (int piece = 0; piece < 2 * NI; ++piece) fetch_piece(kt, piece, page, kdst, vdst);
     };
 
     if (n_kv_tiles > 0) {
@@ -323,12 +337,12 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
       const char* kcur = kBuf ? s_k1 : s_k0;
       const char* vcur = kBuf ? s_v1 : s_v0;
       const bool more = kt + 1 < n_kv_tiles;
-      if (more) {
-        fetch(kt + 1, page_next, kBuf ? s_k0 : s_k1, kBuf ? s_v0 : s_v1);
-        lookup(kt + 2, page_next);
-      }
+      char* knext = kBuf ? s_k0 : s_k1;
+      char* vnext = kBuf ? s_v0 : s_v1;
+      constexpr int kIssueEvery = DS / NI;  // MFMA steps between two staging loads: 2 * DS steps, 2 * NI pieces
 
       const int key0 = kt * kTileN;
+      if (key0 >= wave_max && more) fetch(kt + 1, page_next, knext, vnext);  // no arithmetic to hide the loads behind
       if (key0 < wave_max) {
         // ---- S^T = K Q^T for the two 32-key blocks of the tile ----
         f32x16 s_acc[MB][2];
@@ -350,6 +364,7 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
           for (int t = 0; t < 2 * DS; ++t) {
             const s16x8 ka = __builtin_bit_cast(s16x8, ring[t % kPrefetch]);
             if (t + kPrefetch < 2 * DS) ring[t % kPrefetch] = read_k(t + kPrefetch);
+            if (more && t % kIssueEvery == 0) fetch_piece(kt + 1, t / kIssueEvery, page_next, knext, vnext);
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) s_acc[mb][t / DS] = E::mfma(ka, qreg[mb][t % DS], s_acc[mb][t / DS]);
           }
@@ -380,9 +395,14 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
 #pragma unroll
           for (int x = 1; x < 32; ++x) mx = fmaxf(mx, sc[x]);
           mx = fmaxf(mx, __shfl_xor(mx, 32));
-          const float m_new = fmaxf(m_run[mb], mx * a.qscale);
+          // Lazy running maximum: the reference point m_run only moves when some row's maximum has
+          // grown by more than kMaxSlack (log2 units); until then exp2(s - m_run) may reach
+          // 2^kMaxSlack, harmless in bf16/f16 P and fp32 sums, and the accumulators need no rescale.
+          const float m_cand = mx * a.qscale;
+          const bool moved = __any(m_cand > m_run[mb] + kMaxSlack);
+          const float m_new = moved ? fmaxf(m_run[mb], m_cand) : m_run[mb];
           const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-          const float alpha = fast_exp2(m_run[mb] - m_safe);
+          const float alpha = moved ? fast_exp2(m_run[mb] - m_safe) : 1.f;
           m_run[mb] = m_new;
           float psum = 0.f;
           uint32_t pw[16];
@@ -397,10 +417,12 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
 #pragma unroll
           for (int j = 0; j < 4; ++j)
             p_op[mb][j] = __builtin_bit_cast(s16x8, v4u{pw[4 * j], pw[4 * j + 1], pw[4 * j + 2], pw[4 * j + 3]});
-          l_run[mb] = l_run[mb] * alpha + psum;
-          if (__any(alpha != 1.f)) {
+          if (moved) {
+            l_run[mb] = l_run[mb] * alpha + psum;
 #pragma unroll
             for (int db = 0; db < DB; ++db) o_acc[mb][db] *= alpha;
+          } else {
+            l_run[mb] += psum;
           }
         }
 
@@ -429,6 +451,7 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
         }
       }
 
+      if (more) lookup(kt + 2, page_next);  // page ids for the tile after next; consumed a tile from now
       __builtin_amdgcn_s_waitcnt(0x0F70);  // the rows fetched for the next tile have landed
       __syncthreads();
     };
@@ -463,18 +486,27 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
   }
 }
 
-template <typename E, int D>
-void launch(const PrefillArgs& a0, hipStream_t st) {
+template <typename E, int D, int G>
+void launch_group(const PrefillArgs& a0, hipStream_t st) {
   PrefillArgs a = a0;
-  constexpr int MB = 1;
-  constexpr int BM = kWaves * 32 * MB;
+  constexpr int BM = (kWaves / G) * 32;
   a.n_tiles = (a.Lq + BM - 1) / BM;
-  const int G = a.Hq / a.Hc;
-  dim3 grid(a.Hc, G * a.n_tiles);
+  dim3 grid(a.Hc, a.n_tiles);
   if (a.pd.shift >= 0)
-    hipLaunchKernelGGL((paged_prefill_kernel<E, D, MB, true>), grid, dim3(kThreads), 0, st, a);
+    hipLaunchKernelGGL((paged_prefill_kernel<E, D, G, true>), grid, dim3(kThreads), 0, st, a);
   else
-    hipLaunchKernelGGL((paged_prefill_kernel<E, D, MB, false>), grid, dim3(kThreads), 0, st, a);
+    hipLaunchKernelGGL((paged_prefill_kernel<E, D, G, false>), grid, dim3(kThreads), 0, st, a);
+}
+
+template <typename E, int D>
+int launch(const PrefillArgs& a, hipStream_t st) {
+  switch (a.Hq / a.Hc) {
+    case 1: launch_group<E, D, 1>(a, st); return FP_OK;
+    case 2: launch_group<E, D, 2>(a, st); return FP_OK;
+    case 4: launch_group<E, D, 4>(a, st); return FP_OK;
+    case 8: launch_group<E, D, 8>(a, st); return FP_OK;
+    default: return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill: Hq/Hc = %d (supported: 1, 2, 4, 8)", a.Hq / a.Hc);
+  }
 }
 
 }  // namespace
@@ -501,8 +533,7 @@ extern "C" int fp_paged_prefill(const void* q, int64_t q_stride_row, int64_t q_s
   if (!fp::aligned(q, 16) || !fp::aligned(pool_k, 16) || !fp::aligned(pool_v, 16) || !fp::aligned(out, 8) ||
       (q_stride_row * 2) % 16 || (q_stride_h * 2) % 16 || (out_stride_row * 2) % 8 || (out_stride_h * 2) % 8)
     return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_prefill: q rows must be 16-byte and out rows 8-byte aligned");
-  const int64_t tiles = (static_cast<int64_t>(Lq) + 127) / 128;
-  if (tiles * (Hq / Hc) > 65535) return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill: too many query tiles");
+  if ((static_cast<int64_t>(Lq) + 31) / 32 > 65535) return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill: too many query rows");
 
   PrefillArgs a{static_cast<const char*>(q), q_stride_row * 2, q_stride_h * 2,
                 static_cast<const char*>(pool_k), static_cast<const char*>(pool_v),
@@ -510,10 +541,11 @@ extern "C" int fp_paged_prefill(const void* q, int64_t q_stride_row, int64_t q_s
                 static_cast<char*>(out), out_stride_row * 2, out_stride_h * 2, lse,
                 Lq, Hq, Hc, fp::PageDiv(page_size), n_pages, max_batch, n_slots, scale * kLog2e, 0};
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (dtype == FP_DTYPE_BF16) {
-    if (D == 64) launch<BF16, 64>(a, st); else launch<BF16, 128>(a, st);
-  } else {
-    if (D == 64) launch<F16, 64>(a, st); else launch<F16, 128>(a, st);
-  }
+  int rc;
+  if (dtype == FP_DTYPE_BF16)
+    rc = D == 64 ? launch<BF16, 64>(a, st) : launch<BF16, 128>(a, st);
+  else
+    rc = D == 64 ? launch<F16, 64>(a, st) : launch<F16, 128>(a, st);
+  if (rc != FP_OK) return rc;
   return fp::check_launch("fp_paged_prefill");
 }
