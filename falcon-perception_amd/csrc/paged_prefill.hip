@@ -16,8 +16,9 @@
 //   O^T = V^T P^T: P^T is already in B-operand layout in the S^T accumulators; V^T
 //         comes out of LDS through ds_read_b64_tr_b16, so V is staged row-major like K.
 //   K/V tiles of 64 keys are fetched page by page one tile ahead with global_load_lds
-//   (16 bytes per lane straight into LDS, no staging registers), page ids two tiles ahead,
-//   into a double buffer whose rows are chunk-permuted against bank conflicts.
+//   (16 bytes per lane straight into LDS, no staging registers), page ids two tiles ahead
+//   and turned into row addresses right after the barrier, into a double buffer whose rows
+//   are chunk-permuted against bank conflicts.
 // Rows of one tile may belong to several sequences: the tile is processed one
 // run of equal batch_idx at a time; rows of slot 0 are padding (out 0, lse -inf).
 #include "fp_common.h"
@@ -270,13 +271,16 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
       for (int db = 0; db < DB; ++db) o_acc[mb][db] = kZero16;
     }
 
-    // ---- K/V fetch pipeline: page ids two tiles ahead, rows one tile ahead straight into LDS ----
+    // ---- K/V fetch pipeline ----
+    // Every wavefront stages NI groups of RPI rows of each tile.  Page ids are loaded a tile
+    // before they are needed and turned into row addresses right after a barrier, where every
+    // load of this wavefront has landed anyway; the staging loads themselves then need no wait.
+    // A key that does not exist (past the run's last key, or an unmapped page) reads slot 0:
+    // finite bytes, and every such key is masked.  Tiles past the last one are staged the same
+    // way (all rows from slot 0) so the loop carries no "is there a next tile" branches.
     const int64_t* pt_row = a.page_table + static_cast<int64_t>(sq) * a.pt_row_stride;
-    // Page ids of the rows this lane fetches for the next tile, as loaded (not yet turned into
-    // slots: using them right after the load would make the wavefront wait for every load in
-    // flight, the row fetches included).  A key that does not exist (past the run's last key, or
-    // an unmapped page) reads slot 0: finite bytes, and every such key is masked.
-    int64_t page_next[NI];
+    int64_t page_next[NI];  // page ids of the rows this lane stages next, as loaded
+    int64_t rowbyte[NI];    // byte offset of those rows inside a head's plane
 
     auto key_block = [&](int kpos, int& blkid, int& off) {
       if (kPow2) {  // page size is a power of two: shift and mask, no branch on the page size
@@ -287,87 +291,93 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
         off = kpos - blkid * a.pd.page_size;
       }
     };
-    auto lookup = [&](int kt, int64_t (&page)[NI]) {
+    auto lookup = [&](int kt) {
 #pragma unroll
       for (int i = 0; i < NI; ++i) {
         const int kpos = kt * kTileN + i * kWaves * RPI + st_row0;
         int blkid, off;
         key_block(kpos, blkid, off);
-        page[i] = pt_row[(kpos < kv_max && blkid < a.n_pages) ? blkid : 0];
+        page_next[i] = pt_row[(kpos < kv_max && blkid < a.n_pages) ? blkid : 0];
       }
     };
+    auto resolve = [&](int kt) {  // page_next holds the ids of tile kt
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        const int kpos = kt * kTileN + i * kWaves * RPI + st_row0;
+        int blkid, off;
+        key_block(kpos, blkid, off);
+        const bool ok = kpos < kv_max && blkid < a.n_pages && page_next[i] >= 0 && page_next[i] < a.n_pages;
+        const int slot = ok ? static_cast<int>(page_next[i]) * a.pd.page_size + off : 0;
+        rowbyte[i] = static_cast<int64_t>(slot) * ROWB;
+      }
+    };
+    const char* ksrc = kplane + k_src_off;
+    const char* vsrc = vplane + v_src_off;
     // One staging load: piece 2 * i is the K load of row group i, piece 2 * i + 1 its V load.
-    // The pieces of the next tile are issued one at a time between the MFMAs of the current
-    // tile: the CU moves 64 bytes per cycle from L2 towards LDS, and a burst of all pieces
-    // from all wavefronts at once would hold each wavefront at its load instructions.
-    auto fetch_piece = [&](int kt, int piece, const int64_t (&page)[NI], char* kdst, char* vdst) {
+    auto fetch_piece = [&](int piece, char* kdst, char* vdst) {
       const int i = piece >> 1;
-      const int kpos = kt * kTileN + i * kWaves * RPI + st_row0;
-      int blkid, off;
-      key_block(kpos, blkid, off);
-      const bool ok = kpos < kv_max && blkid < a.n_pages && page[i] >= 0 && page[i] < a.n_pages;
-      const int slot = ok ? static_cast<int>(page[i]) * a.pd.page_size + off : 0;
-      const int64_t rowbyte = static_cast<int64_t>(slot) * ROWB;
       const int group = (i * kWaves + wave) * RPI * ROWB;  // wavefront-uniform LDS offset
       if ((piece & 1) == 0)
-        __builtin_amdgcn_global_load_lds(
-            (const __attribute__((address_space(1))) void*)(kplane + rowbyte + k_src_off),
-            (__attribute__((address_space(3))) void*)(kdst + group), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(ksrc + rowbyte[i]),
+                                         (__attribute__((address_space(3))) void*)(kdst + group), 16, 0, 0);
       else
-        __builtin_amdgcn_global_load_lds(
-            (const __attribute__((address_space(1))) void*)(vplane + rowbyte + v_src_off),
-            (__attribute__((address_space(3))) void*)(vdst + group), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(vsrc + rowbyte[i]),
+                                         (__attribute__((address_space(3))) void*)(vdst + group), 16, 0, 0);
     };
-    auto fetch = [&](int kt, const int64_t (&page)[NI], char* kdst, char* vdst) {
+    auto fetch = [&](char* kdst, char* vdst) {
 #pragma unroll
-      for (int piece = 0; piece < 2 * NI; ++piece) fetch_piece(kt, piece, page, kdst, vdst);
+      for (int piece = 0; piece < 2 * NI; ++piece) fetch_piece(piece, kdst, vdst);
     };
 
-    if (n_kv_tiles > 0) {
-      lookup(0, page_next);
-      fetch(0, page_next, s_k0, s_v0);
-      lookup(1, page_next);
-    }
+    // per-lane LDS offsets of the operand reads, the same for every tile and buffer
+    int kofs[DS], vofs[DB];
+#pragma unroll
+    for (int ds = 0; ds < DS; ++ds) kofs[ds] = ln * ROWB + (((2 * ds) ^ ksel) * 16);
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+      vofs[db] = (half * 4 + (bi >> 2)) * ROWB + (bi & 3) * 8 + ((2 * db + vsel) % R32) * 32;
+
+    lookup(0);
+    resolve(0);
+    fetch(s_k0, s_v0);
+    lookup(1);
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's rows have landed in LDS
     __syncthreads();
 
-    // one tile: start the fetch of the next tile into the other buffer, then work on this one
+    // one tile: stage tile kt + 1 into the other buffer while working on tile kt
     auto tile_step = [&](auto parity, int kt) {
       constexpr int kBuf = decltype(parity)::value;
       const char* kcur = kBuf ? s_k1 : s_k0;
       const char* vcur = kBuf ? s_v1 : s_v0;
-      const bool more = kt + 1 < n_kv_tiles;
-      char* knext = kBuf ? s_k0 : s_k1;
-      char* vnext = kBuf ? s_v0 : s_v1;
+      char* k1 = kBuf ? s_k0 : s_k1;
+      char* v1 = kBuf ? s_v0 : s_v1;
       constexpr int kIssueEvery = DS / NI;  // MFMA steps between two staging loads: 2 * DS steps, 2 * NI pieces
 
       const int key0 = kt * kTileN;
-      if (key0 >= wave_max && more) fetch(kt + 1, page_next, knext, vnext);  // no arithmetic to hide the loads behind
-      if (key0 < wave_max) {
+      const bool work = key0 < wave_max;
+      resolve(kt + 1);
+      lookup(kt + 2);
+      if (!work) fetch(k1, v1);  // no arithmetic to hide the loads behind
+
+      if (work) {
+        f32x16 s_acc[MB][2];  // written by the first MFMA of each block, which starts from zero
         // ---- S^T = K Q^T for the two 32-key blocks of the tile ----
-        f32x16 s_acc[MB][2];
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-          for (int kb = 0; kb < 2; ++kb) s_acc[mb][kb] = kZero16;
         // LDS operands are read kPrefetch steps ahead of the MFMA that consumes them
-        {
-          const char* krow = kcur + ln * ROWB;
-          auto read_k = [&](int t) {
-            const int kb = t / DS, ds = t % DS;
-            return *reinterpret_cast<const v4u*>(krow + kb * 32 * ROWB + (((2 * ds) ^ ksel) * 16));
-          };
-          v4u ring[kPrefetch];
+        auto read_k = [&](int t) {
+          const int kb = t / DS, ds = t % DS;
+          return *reinterpret_cast<const v4u*>(kcur + kofs[ds] + kb * 32 * ROWB);
+        };
+        v4u ring[kPrefetch];
 #pragma unroll
-          for (int t = 0; t < kPrefetch; ++t) ring[t] = read_k(t);
+        for (int t = 0; t < kPrefetch; ++t) ring[t] = read_k(t);
 #pragma unroll
-          for (int t = 0; t < 2 * DS; ++t) {
-            const s16x8 ka = __builtin_bit_cast(s16x8, ring[t % kPrefetch]);
-            if (t + kPrefetch < 2 * DS) ring[t % kPrefetch] = read_k(t + kPrefetch);
-            if (more && t % kIssueEvery == 0) fetch_piece(kt + 1, t / kIssueEvery, page_next, knext, vnext);
+        for (int t = 0; t < 2 * DS; ++t) {
+          const s16x8 ka = __builtin_bit_cast(s16x8, ring[t % kPrefetch]);
+          if (t + kPrefetch < 2 * DS) ring[t % kPrefetch] = read_k(t + kPrefetch);
+          if (t % kIssueEvery == 0) fetch_piece(t / kIssueEvery, k1, v1);
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb) s_acc[mb][t / DS] = E::mfma(ka, qreg[mb][t % DS], s_acc[mb][t / DS]);
-          }
+          for (int mb = 0; mb < MB; ++mb)
+            s_acc[mb][t / DS] = E::mfma(ka, qreg[mb][t % DS], t % DS == 0 ? kZero16 : s_acc[mb][t / DS]);
         }
 
         // ---- online softmax, one query per lane ----
@@ -383,6 +393,7 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
 #pragma unroll
             for (int i = 0; i < 16; ++i) sc[kb * 16 + i] = s_acc[mb][kb][i];
           if (need_mask) {
+            asm volatile("");  // keeps this a branch: turned into selects it would run on every tile
             // register i of block kb is key kb*32 + (i/4)*8 + half*4 + i%4 of the tile
             const int rel = lim[mb] - key0 - half * 4;
 #pragma unroll
@@ -418,6 +429,7 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
           for (int j = 0; j < 4; ++j)
             p_op[mb][j] = __builtin_bit_cast(s16x8, v4u{pw[4 * j], pw[4 * j + 1], pw[4 * j + 2], pw[4 * j + 3]});
           if (moved) {
+            asm volatile("");  // likewise: the rescale is rare and must not run unconditionally
             l_run[mb] = l_run[mb] * alpha + psum;
 #pragma unroll
             for (int db = 0; db < DB; ++db) o_acc[mb][db] *= alpha;
@@ -430,10 +442,9 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
         {
           // step t = (j, db): this lane names the chunk (key = base + bi / 4, d = dblock + 4 * (bi % 4))
           // and receives d = dblock + bi for keys base .. base + 3, once for each half of the 16 keys
-          const char* vrow = vcur + (half * 4 + (bi >> 2)) * ROWB + (bi & 3) * 8;
           auto read_v = [&](int t, s16x4& lo, s16x4& hi) {
             const int j = t / DB, db = t % DB;
-            const char* p0 = vrow + ((j >> 1) * 32 + (j & 1) * 16) * ROWB + ((2 * db + vsel) % R32) * 32;
+            const char* p0 = vcur + vofs[db] + ((j >> 1) * 32 + (j & 1) * 16) * ROWB;
             lo = lds_read_tr(p0);
             hi = lds_read_tr(p0 + 8 * ROWB);
           };
@@ -451,8 +462,7 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
         }
       }
 
-      if (more) lookup(kt + 2, page_next);  // page ids for the tile after next; consumed a tile from now
-      __builtin_amdgcn_s_waitcnt(0x0F70);  // the rows fetched for the next tile have landed
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // this wavefront's share of tile kt + 1 has landed
       __syncthreads();
     };
 
