@@ -45,7 +45,7 @@ DTYPES = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
 
 # HBM bytes per launch of paged_decode_kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # (profiles/), scaled by the same counters on a plain copy of known size; None = not measured
-TRAFFIC_BYTES = {"cfg2": 671.7e6}  # profiles/paged_decode_cfg2_hbm_traffic.md
+TRAFFIC_BYTES = {"cfg2": 671.9e6}  # profiles/paged_decode_cfg2_hbm_traffic.md
 
 
 @dataclass
@@ -370,16 +370,19 @@ def append_gather_rates(steps: int = 20, T: int = 32768, H: int = 16, D: int = 1
             "kv_gather_frac_of_peak": bytes_g / (ms_g * 1e-3) / 1e9 / HBM_PEAK_GBPS}
 
 
-def prefill_rate(steps: int = 10) -> dict:
+def prefill_rate(steps: int = 10, name: str = "cfg3") -> dict:
     """Chunked prefill at BASELINE configs[2]: append the 512-token chunks, attend over the paged prefix."""
-    case = make_prefill_case("cfg3")
+    case = make_prefill_case(name)
     case.append()
     for _ in range(3):
         case.attend()
     ms = event_ms(case.attend, steps)
     ms_a = event_ms(case.append, steps)
     tf = case.flops() / (ms * 1e-3) / 1e12
-    return {"workload": "cfg3: 8 sequences, paged prefix U[256,4096], 512-token chunk each, 16 q / 8 kv heads, D 128",
+    what = {"cfg3": "cfg3: 8 sequences, paged prefix U[256,4096], 512-token chunk each, 16 q / 8 kv heads, D 128",
+            "cfg3w": "cfg3w: the same 8 sequences prefilled whole (prefix + chunk rows in one step, prefix rows see "
+                     "their whole image span), 16 q / 8 kv heads, D 128"}[name]
+    return {"workload": what, "query_rows": int(case.q.shape[2]),
             "paged_prefill_ms": ms, "tflops": tf, "frac_of_bf16_mfma_peak": tf / MFMA_BF16_PEAK_TFLOPS,
             "chunk_append_ms": ms_a, "flops": case.flops()}
 
@@ -440,6 +443,8 @@ def main() -> int:
                     help="also run a plain 1 GiB elementwise copy (x * 2) a few times, so a rocprofv3 --pmc run of this "
                          "command holds a kernel of known traffic next to the decode kernel")
     ap.add_argument("--hbm-budget-gb", type=float, default=None, help="pool size for cfg5")
+    ap.add_argument("--prefill-only", default=None, choices=sorted(PREFILL_WORKLOADS),
+                    help="time only the chunked-prefill attention of this workload and print its JSON (for profiling)")
     args = ap.parse_args()
 
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -453,6 +458,9 @@ def main() -> int:
     from falcon_perception_amd import _native
 
     _native.lib()  # fail loudly if the HIP library is not built
+    if args.prefill_only:
+        print(json.dumps(prefill_rate(max(args.steps, 1), args.prefill_only)))
+        return 0
     case = make_decode_case(args.workload, hbm_budget_gb=args.hbm_budget_gb)
     c = case.cfg
 
