@@ -111,6 +111,22 @@ class DecodeCase:
                                 split_tokens=self.split_tokens, workspace=self.workspace,
                                 out=self.out, lse=self.lse, k_new=self.k_new, v_new=self.v_new)
 
+    def run_fused_gated(self):
+        """run_fused plus the caller's post-attention sink gate (reference model.py:122-127) inside the
+        merge pass, written in the [B, 1, Hq * D] layout of the output projection."""
+        from falcon_perception_amd import ops
+
+        c = self.cfg
+        if "sinks" not in self.extra:
+            self.extra["sinks"] = torch.linspace(-2.0, 2.0, c["Hq"], device=self.q.device)
+            self.extra["flat"] = torch.empty((c["B"], 1, c["Hq"] * c["D"]), dtype=self.q.dtype, device=self.q.device)
+        out = self.extra["flat"].view(c["B"], 1, c["Hq"], c["D"]).permute(0, 2, 1, 3)
+        return ops.paged_decode(self.q, self.pool_k, self.pool_v, self.cache.page_table, self.batch_idx,
+                                self.input_pos, self.page_size, self.max_context,
+                                split_tokens=self.split_tokens, workspace=self.workspace,
+                                out=out, lse=self.lse, k_new=self.k_new, v_new=self.v_new,
+                                sinks=self.extra["sinks"])
+
     # ---- algorithmic traffic (bytes) --------------------------------------
     def bytes_append(self):
         c = self.cfg
@@ -474,6 +490,7 @@ def main() -> int:
 
     ms_step = time_steps(case.run_fused, args.steps, args.warmup)
     ms_separate = time_steps(case.run, args.steps, args.warmup)
+    ms_gated = time_steps(case.run_fused_gated, args.steps, args.warmup)
     ms_graph = graph_ms(case.run_fused, args.steps)
     ms_decode = event_ms(case.attend, args.steps)
     ms_partial = event_ms(lambda: case.attend("partial"), args.steps)  # the dominant kernel alone
@@ -501,6 +518,7 @@ def main() -> int:
         "decode_tok_s_model": c["B"] / (ms_step * 1e-3) / MODEL_LAYERS,
         "step": "fp_paged_decode_append (append fused into the split-K pass) + merge pass",
         "ms_per_step_separate_append": ms_separate,
+        "ms_per_step_with_sink_gate": ms_gated,  # same step, sigmoid(lse - sink) gate + [B,1,H*D] layout in the merge
         "value_separate_append": alg_step / (ms_separate * 1e-3) / 1e9,
         "ms_per_step_hip_graph": ms_graph,
         "value_hip_graph": alg_step / (ms_graph * 1e-3) / 1e9,

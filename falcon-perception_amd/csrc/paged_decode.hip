@@ -45,6 +45,7 @@ struct DecodeArgs {
   char* out;
   int64_t os_b, os_h;  // bytes
   float* lse;
+  const float* sinks;  // optional [Hq]: out is multiplied by sigmoid(lse - sinks[h])
   float* ws_acc;  // [B, Hq, n_splits, D]
   float* ws_ml;   // [B, Hq, n_splits, 2]
   int Hq, Hc;
@@ -88,6 +89,7 @@ struct F32 {
     f[3] = __uint_as_float(r.w);
   }
   static __device__ __forceinline__ void store(char* p, float v) { *reinterpret_cast<float*>(p) = v; }
+  static __device__ __forceinline__ float round(float v) { return v; }
 };
 // bf16 / f16: q.k on the packed pairs with v_dot2 (fp32 accumulate), no conversion of K
 struct BF16 {
@@ -115,6 +117,7 @@ struct BF16 {
   static __device__ __forceinline__ void store(char* p, float v) {
     *reinterpret_cast<__hip_bfloat16*>(p) = __float2bfloat16(v);
   }
+  static __device__ __forceinline__ float round(float v) { return __bfloat162float(__float2bfloat16(v)); }
 };
 struct F16 {
   using type = __half;
@@ -140,11 +143,22 @@ struct F16 {
     }
   }
   static __device__ __forceinline__ void store(char* p, float v) { *reinterpret_cast<__half*>(p) = __float2half(v); }
+  static __device__ __forceinline__ float round(float v) { return __half2float(__float2half(v)); }
 };
 
 // K and V are streamed once: non-temporal loads keep them from displacing the caches
 __device__ __forceinline__ v4u stream_load(const char* p) {
   return __builtin_nontemporal_load(reinterpret_cast<const v4u*>(p));
+}
+
+// Attention-sink gate of the caller's post-attention step (model.py:122-128), applied where the
+// output row and its lse are final: the reference multiplies the attention output, already rounded
+// to the model dtype, by sigmoid(lse - sinks[h]) in fp32 and rounds again.
+template <typename E>
+__device__ __forceinline__ float sink_gate(float o, float lse_nat, const float* sinks, int hq) {
+  if (sinks == nullptr) return o;
+  const float g = 1.f / (1.f + __expf(sinks[hq] - lse_nat));
+  return E::round(o) * g;
 }
 
 // ---- cross-lane helpers ---------------------------------------------------
@@ -428,8 +442,9 @@ __global__ __launch_bounds__(kThreads) void paged_decode_kernel(const DecodeArgs
     }
     const int hq = hc * G + g;
     if (kDirect) {
-      E::store(a.out + b * a.os_b + hq * a.os_h + d * sizeof(typename E::type), num / den);
-      if (d == 0) a.lse[static_cast<int64_t>(b) * a.Hq + hq] = (mn + log2f(den)) * kLn2;
+      const float lse_nat = (mn + log2f(den)) * kLn2;
+      E::store(a.out + b * a.os_b + hq * a.os_h + d * sizeof(typename E::type), sink_gate<E>(num / den, lse_nat, a.sinks, hq));
+      if (d == 0) a.lse[static_cast<int64_t>(b) * a.Hq + hq] = lse_nat;
     } else {
       const int64_t p = (static_cast<int64_t>(b) * a.Hq + hq) * a.n_splits + split;
       a.ws_acc[p * D + d] = num;
@@ -460,14 +475,14 @@ __global__ __launch_bounds__(64) void paged_decode_merge_kernel(const DecodeArgs
   float den = 0.f;
   for (int s = 0; s < ns; ++s) den += a.ws_ml[(p0 + s) * 2 + 1] * fast_exp2(a.ws_ml[(p0 + s) * 2] - ms);
 
+  const float lse_nat = ns > 0 ? (mn + log2f(den)) * kLn2 : -INFINITY;
   for (int d = threadIdx.x; d < D; d += 64) {
     float num = 0.f;
     for (int s = 0; s < ns; ++s) num += a.ws_acc[(p0 + s) * D + d] * fast_exp2(a.ws_ml[(p0 + s) * 2] - ms);
     const float o = ns > 0 ? num / den : 0.f;
-    E::store(a.out + b * a.os_b + hq * a.os_h + d * sizeof(typename E::type), o);
+    E::store(a.out + b * a.os_b + hq * a.os_h + d * sizeof(typename E::type), sink_gate<E>(o, lse_nat, a.sinks, hq));
   }
-  if (threadIdx.x == 0)
-    a.lse[static_cast<int64_t>(b) * a.Hq + hq] = ns > 0 ? (mn + log2f(den)) * kLn2 : -INFINITY;
+  if (threadIdx.x == 0) a.lse[static_cast<int64_t>(b) * a.Hq + hq] = lse_nat;
 }
 
 constexpr int kPhasePartial = 1;
@@ -561,7 +576,7 @@ struct NewRows {
 int decode_entry(int phases, const NewRows* fresh, const void* q, int64_t q_stride_b, int64_t q_stride_h, const void* pool_k,
                  const void* pool_v, const int64_t* page_table, int64_t pt_row_stride,
                  const int64_t* batch_idx, const void* input_pos, int pos_index_type,
-                 void* out, int64_t out_stride_b, int64_t out_stride_h, float* lse,
+                 void* out, int64_t out_stride_b, int64_t out_stride_h, float* lse, const float* sinks,
                  void* workspace, int64_t workspace_bytes, int32_t B, int32_t Hq, int32_t Hc,
                  int32_t D, int32_t page_size, int32_t n_pages, int32_t max_batch,
                  int64_t n_slots, int32_t max_context, int32_t split_tokens, float scale,
@@ -599,7 +614,7 @@ int decode_entry(int phases, const NewRows* fresh, const void* q, int64_t q_stri
   DecodeArgs a{static_cast<const char*>(q), q_stride_b * eb, q_stride_h * eb,
                static_cast<const char*>(pool_k), static_cast<const char*>(pool_v),
                page_table, pt_row_stride, batch_idx, input_pos, pos_index_type == FP_INDEX_I64,
-               static_cast<char*>(out), out_stride_b * eb, out_stride_h * eb, lse,
+               static_cast<char*>(out), out_stride_b * eb, out_stride_h * eb, lse, sinks,
                nullptr, nullptr, Hq, Hc, fp::PageDiv(page_size), n_pages, max_batch, n_slots,
                max_context, split_tokens, ns, scale * kLog2e,  // scores are kept in log2 units
                nullptr, nullptr, 0, 0, 0, 0};
@@ -641,12 +656,13 @@ int decode_entry(int phases, const NewRows* fresh, const void* q, int64_t q_stri
   const void *q, int64_t q_stride_b, int64_t q_stride_h, const void *pool_k, const void *pool_v,          \
       const int64_t *page_table, int64_t pt_row_stride, const int64_t *batch_idx, const void *input_pos,  \
       int pos_index_type, void *out, int64_t out_stride_b, int64_t out_stride_h, float *lse,              \
+      const float *sinks,                                                                                 \
       void *workspace, int64_t workspace_bytes, int32_t B, int32_t Hq, int32_t Hc, int32_t D,             \
       int32_t page_size, int32_t n_pages, int32_t max_batch, int64_t n_slots, int32_t max_context,        \
       int32_t split_tokens, float scale, int dtype, void *stream
 #define FP_DECODE_ARGS                                                                                     \
   q, q_stride_b, q_stride_h, pool_k, pool_v, page_table, pt_row_stride, batch_idx, input_pos,             \
-      pos_index_type, out, out_stride_b, out_stride_h, lse, workspace, workspace_bytes, B, Hq, Hc, D,     \
+      pos_index_type, out, out_stride_b, out_stride_h, lse, sinks, workspace, workspace_bytes, B, Hq, Hc, D, \
       page_size, n_pages, max_batch, n_slots, max_context, split_tokens, scale, dtype, stream
 
 extern "C" int fp_paged_decode(FP_DECODE_PARAMS) {

@@ -56,6 +56,7 @@ struct PrefillArgs {
   char* out;
   int64_t os_row, os_h;  // bytes
   float* lse;            // [Hq, Lq]
+  const float* sinks;    // optional [Hq]: out is multiplied by sigmoid(lse - sinks[h])
   int Lq, Hq, Hc;
   fp::PageDiv pd;
   int n_pages, max_batch;
@@ -77,6 +78,7 @@ struct BF16 {
     const bf16x2 v = {static_cast<__bf16>(lo), static_cast<__bf16>(hi)};
     return __builtin_bit_cast(uint32_t, v);
   }
+  static __device__ __forceinline__ float round(float x) { return static_cast<float>(static_cast<__bf16>(x)); }
 };
 struct F16 {
   using vec8 = f16x8;
@@ -91,6 +93,7 @@ struct F16 {
     const f16x2 v = {static_cast<_Float16>(lo), static_cast<_Float16>(hi)};
     return __builtin_bit_cast(uint32_t, v);
   }
+  static __device__ __forceinline__ float round(float x) { return static_cast<float>(static_cast<_Float16>(x)); }
 };
 
 constexpr f32x16 kZero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
@@ -478,19 +481,24 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
       const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
       if (!active[mb]) continue;
       char* o = a.out + row[mb] * a.os_row + hq * a.os_h;
+      const float lse_nat = l_tot > 0.f ? (m_run[mb] + log2f(l_tot)) * kLn2 : -INFINITY;
+      // attention-sink gate of the caller's post-attention step (model.py:122-128): the output,
+      // rounded to the model dtype, times sigmoid(lse - sinks[h]) in fp32, rounded again
+      const bool gated = a.sinks != nullptr;
+      const float gate = gated ? 1.f / (1.f + __expf(a.sinks[hq] - lse_nat)) : 1.f;
+      auto fin = [&](float x) { return gated ? E::round(x * inv) * gate : x * inv; };
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
 #pragma unroll
         for (int i4 = 0; i4 < 4; ++i4) {
           // registers 4*i4 .. 4*i4+3 hold d = db*32 + i4*8 + half*4 + 0..3
           const int d = db * 32 + i4 * 8 + half * 4;
-          const uint32_t w0 = E::pack2(o_acc[mb][db][i4 * 4 + 0] * inv, o_acc[mb][db][i4 * 4 + 1] * inv);
-          const uint32_t w1 = E::pack2(o_acc[mb][db][i4 * 4 + 2] * inv, o_acc[mb][db][i4 * 4 + 3] * inv);
+          const uint32_t w0 = E::pack2(fin(o_acc[mb][db][i4 * 4 + 0]), fin(o_acc[mb][db][i4 * 4 + 1]));
+          const uint32_t w1 = E::pack2(fin(o_acc[mb][db][i4 * 4 + 2]), fin(o_acc[mb][db][i4 * 4 + 3]));
           *reinterpret_cast<uint2*>(o + d * 2) = uint2{w0, w1};
         }
       }
-      if (half == 0)
-        a.lse[static_cast<int64_t>(hq) * a.Lq + row[mb]] = l_tot > 0.f ? (m_run[mb] + log2f(l_tot)) * kLn2 : -INFINITY;
+      if (half == 0) a.lse[static_cast<int64_t>(hq) * a.Lq + row[mb]] = lse_nat;
     }
     run0 = run1;
   }
@@ -524,7 +532,8 @@ int launch(const PrefillArgs& a, hipStream_t st) {
 extern "C" int fp_paged_prefill(const void* q, int64_t q_stride_row, int64_t q_stride_h, const void* pool_k,
                                 const void* pool_v, const int64_t* page_table, int64_t pt_row_stride,
                                 const int64_t* batch_idx, const int32_t* row_limit, void* out,
-                                int64_t out_stride_row, int64_t out_stride_h, float* lse, int32_t Lq, int32_t Hq,
+                                int64_t out_stride_row, int64_t out_stride_h, float* lse, const float* sinks,
+                                int32_t Lq, int32_t Hq,
                                 int32_t Hc, int32_t D, int32_t page_size, int32_t n_pages, int32_t max_batch,
                                 int64_t n_slots, float scale, int dtype, void* stream) {
   if (dtype != FP_DTYPE_BF16 && dtype != FP_DTYPE_F16)
@@ -548,7 +557,7 @@ extern "C" int fp_paged_prefill(const void* q, int64_t q_stride_row, int64_t q_s
   PrefillArgs a{static_cast<const char*>(q), q_stride_row * 2, q_stride_h * 2,
                 static_cast<const char*>(pool_k), static_cast<const char*>(pool_v),
                 page_table, pt_row_stride, batch_idx, row_limit,
-                static_cast<char*>(out), out_stride_row * 2, out_stride_h * 2, lse,
+                static_cast<char*>(out), out_stride_row * 2, out_stride_h * 2, lse, sinks,
                 Lq, Hq, Hc, fp::PageDiv(page_size), n_pages, max_batch, n_slots, scale * kLog2e, 0};
   hipStream_t st = static_cast<hipStream_t>(stream);
   int rc;

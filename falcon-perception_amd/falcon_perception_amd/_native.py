@@ -42,7 +42,7 @@ SIGNATURES = {
     "fp_paged_decode": (c_int, [
         c_void_p, c_int64, c_int64, c_void_p, c_void_p,
         c_void_p, c_int64, c_void_p, c_void_p, c_int,
-        c_void_p, c_int64, c_int64, c_void_p,
+        c_void_p, c_int64, c_int64, c_void_p, c_void_p,
         c_void_p, c_int64,
         c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
         c_int64, c_int32, c_int32, c_float, c_int, c_void_p]),
@@ -53,7 +53,7 @@ SIGNATURES = {
     "fp_paged_prefill": (c_int, [
         c_void_p, c_int64, c_int64, c_void_p, c_void_p,
         c_void_p, c_int64, c_void_p, c_void_p,
-        c_void_p, c_int64, c_int64, c_void_p,
+        c_void_p, c_int64, c_int64, c_void_p, c_void_p,
         c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
         c_int64, c_float, c_int, c_void_p]),
 }

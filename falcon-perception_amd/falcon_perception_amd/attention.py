@@ -159,14 +159,18 @@ def _result(out: Tensor, lse: Tensor, return_aux, return_lse: bool):
 
 def compiled_flex_attn_decode(q: Tensor, k: Tensor, v: Tensor, score_mod=None, block_mask=None,
                               scale: float | None = None, enable_gqa: bool = False,
-                              return_lse: bool = False, kernel_options=None, *, return_aux=None):
+                              return_lse: bool = False, kernel_options=None, *, return_aux=None,
+                              sinks: Tensor | None = None):
     """Decode attention, one query token per sequence (`attention.py:17`, `model.py:156-162`).
 
     q [B, Hq, 1, D]; k, v are the pool views `PagedKVCache.insert_kv` returned,
     [1, Hc, n_slots, D].  `kernel_options` are Triton tuning knobs of the reference
-    and are ignored.
+    and are ignored.  `sinks` [Hq] float32 (not an argument of the reference's callable) applies
+    the sink gate of `Attention._post_attention` (`model.py:122-126`) to the returned output.
     """
     if not isinstance(block_mask, PagedDecodeMask):
+        if sinks is not None:
+            raise RuntimeError("the fused sink gate needs a mask made by PagedKVCache")
         return _foreign("decode", q, k, v, dict(score_mod=score_mod, block_mask=block_mask, scale=scale,
                                                 enable_gqa=enable_gqa, return_lse=return_lse,
                                                 kernel_options=kernel_options, return_aux=return_aux))
@@ -183,13 +187,15 @@ def compiled_flex_attn_decode(q: Tensor, k: Tensor, v: Tensor, score_mod=None, b
         cache.page_size, block_mask.max_context, scale=scale,
         workspace=cache.decode_workspace(q.shape[0], q.shape[1], q.shape[3], block_mask.max_context, k.shape[1]),
         split_tokens=cache.decode_split_tokens(q.shape[0], k.shape[1], block_mask.max_context),
+        sinks=sinks,
     )
     return _result(out, lse, return_aux, return_lse)
 
 
 def compiled_flex_attn_prefill(q: Tensor, k: Tensor, v: Tensor, score_mod=None, block_mask=None,
                                scale: float | None = None, enable_gqa: bool = False,
-                               return_lse: bool = False, kernel_options=None, *, return_aux=None):
+                               return_lse: bool = False, kernel_options=None, *, return_aux=None,
+                               sinks: Tensor | None = None):
     """Prefill attention over the paged cache under the hybrid mask (`attention.py:18`).
 
     q [1, Hq, L, D] packed rows.  Keys and values are read from the pages that
@@ -198,6 +204,8 @@ def compiled_flex_attn_prefill(q: Tensor, k: Tensor, v: Tensor, score_mod=None, 
     already lives in pages attends over prefix and chunk alike.
     """
     if not isinstance(block_mask, HybridPrefillMask):
+        if sinks is not None:
+            raise RuntimeError("the fused sink gate needs a mask made by PagedKVCache")
         return _foreign("prefill", q, k, v, dict(score_mod=score_mod, block_mask=block_mask, scale=scale,
                                                  enable_gqa=enable_gqa, return_lse=return_lse,
                                                  kernel_options=kernel_options, return_aux=return_aux))
@@ -211,7 +219,7 @@ def compiled_flex_attn_prefill(q: Tensor, k: Tensor, v: Tensor, score_mod=None, 
     pool_v = cache.kv_cache[step.layer_id, 1, 0]
     out, lse = ops.paged_prefill(
         q, pool_k, pool_v, cache.page_table, step.batch_idx,
-        block_mask.row_limit(step.input_pos), cache.page_size, scale=scale,
+        block_mask.row_limit(step.input_pos), cache.page_size, scale=scale, sinks=sinks,
     )
     return _result(out, lse, return_aux, return_lse)
 

@@ -101,12 +101,25 @@ def decode_workspace_bytes(B: int, Hq: int, D: int, max_context: int, split_toke
     return n
 
 
+def _sinks_ptr(sinks: Tensor | None, Hq: int, device) -> int | None:
+    if sinks is None:
+        return None
+    N.require_cuda(sinks)
+    if sinks.dtype != torch.float32 or sinks.shape != (Hq,) or not sinks.is_contiguous() or sinks.device != device:
+        raise RuntimeError("sinks must be a contiguous float32 tensor of shape [Hq] on the device of q")
+    return sinks.data_ptr()
+
+
 def paged_decode(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor, batch_idx: Tensor,
                  input_pos: Tensor, page_size: int, max_context: int, *, scale: float | None = None,
                  split_tokens: int = 0, workspace: Tensor | None = None,
                  out: Tensor | None = None, lse: Tensor | None = None, phase: str = "both",
-                 k_new: Tensor | None = None, v_new: Tensor | None = None) -> tuple[Tensor, Tensor]:
+                 k_new: Tensor | None = None, v_new: Tensor | None = None,
+                 sinks: Tensor | None = None) -> tuple[Tensor, Tensor]:
     """Single-query paged attention.  q [B, Hq, 1, D]; pools [Hc, N, D]; returns out [B, Hq, 1, D], lse [B, Hq, 1].
+
+    With `sinks` [Hq] float32 the output is gated as the reference's `_post_attention` does
+    (model.py:122-128): out * sigmoid(lse - sinks[h]); lse is returned ungated.
 
     With `k_new`, `v_new` [B, Hc, 1, D] the call is the whole decode step: the rows are appended at
     `input_pos` (as `kv_append` with clamp would) and attended over in the same launch.
@@ -136,6 +149,7 @@ def paged_decode(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor, 
         lse = torch.empty((B, Hq, 1), dtype=torch.float32, device=q.device)
     if out.stride(3) != 1 or not lse.is_contiguous() or lse.dtype != torch.float32:
         raise RuntimeError("out rows must be dense and lse contiguous float32")
+    sinks_ptr = _sinks_ptr(sinks, Hq, q.device)
     entry = {"both": "fp_paged_decode", "partial": "fp_paged_decode_partial", "merge": "fp_paged_decode_merge"}[phase]
     fresh = ()
     if k_new is not None or v_new is not None:
@@ -152,7 +166,7 @@ def paged_decode(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor, 
         q.data_ptr(), q.stride(0), q.stride(1), pool_k.data_ptr(), pool_v.data_ptr(),
         page_table.data_ptr(), page_table.stride(0), batch_idx.data_ptr(),
         input_pos.data_ptr(), N.index_code(input_pos),
-        out.data_ptr(), out.stride(0), out.stride(1), lse.data_ptr(),
+        out.data_ptr(), out.stride(0), out.stride(1), lse.data_ptr(), sinks_ptr,
         workspace.data_ptr() if workspace is not None else None,
         workspace.numel() * workspace.element_size() if workspace is not None else 0,
         B, Hq, Hc, D, page_size, page_table.shape[1], page_table.shape[0],
@@ -176,9 +190,11 @@ def hybrid_row_limits(input_ids: Tensor, soi_id: int, eoi_id: int) -> Tensor:
 
 def paged_prefill(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor, batch_idx: Tensor,
                   row_limit: Tensor, page_size: int, *, scale: float | None = None,
-                  out: Tensor | None = None, lse: Tensor | None = None) -> tuple[Tensor, Tensor]:
+                  out: Tensor | None = None, lse: Tensor | None = None,
+                  sinks: Tensor | None = None) -> tuple[Tensor, Tensor]:
     """Chunked-prefill attention over the paged cache.  q [1, Hq, Lq, D]; row r sees keys
-    0..row_limit[r]-1 of sequence batch_idx[r]; returns out like q, lse [1, Hq, Lq]."""
+    0..row_limit[r]-1 of sequence batch_idx[r]; returns out like q, lse [1, Hq, Lq].
+    `sinks` [Hq] float32 gates the output as in `paged_decode`."""
     N.require_cuda(q, pool_k, pool_v, page_table, batch_idx, row_limit, out, lse)
     one, Hq, Lq, D = q.shape
     if one != 1:
@@ -205,7 +221,7 @@ def paged_prefill(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor,
         q.data_ptr(), q.stride(2), q.stride(1), pool_k.data_ptr(), pool_v.data_ptr(),
         page_table.data_ptr(), page_table.stride(0), batch_idx.data_ptr(),
         row_limit.data_ptr(), out.data_ptr(), out.stride(2), out.stride(1), lse.data_ptr(),
-        Lq, Hq, Hc, D, page_size, page_table.shape[1], page_table.shape[0], n_slots,
+        _sinks_ptr(sinks, Hq, q.device), Lq, Hq, Hc, D, page_size, page_table.shape[1], page_table.shape[0], n_slots,
         scale, N.dtype_code(q.dtype), N.stream_ptr(q.device))
     N.check(rc, "fp_paged_prefill")
     return out, lse

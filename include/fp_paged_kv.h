@@ -147,6 +147,11 @@ int64_t fp_paged_decode_workspace_bytes(int32_t B, int32_t Hq, int32_t D,
  *   input_pos[B] int32/int64: sequence b attends logical positions 0..input_pos[b]
  *   out      [B, Hq, 1, D] same dtype as q, element strides (b, h)
  *   lse      [B, Hq] float32, natural log of the softmax denominator
+ *   sinks    NULL, or [Hq] float32: out is multiplied by sigmoid(lse - sinks[h]), the
+ *            attention-sink gate of Attention._post_attention (model.py:122-128), with the
+ *            reference's rounding (attention output rounded to the dtype, product rounded again);
+ *            lse is returned ungated.  With strides (Hq * D, D) out is then the [B, 1, Hq * D]
+ *            row the reference's output projection takes (model.py:127-128)
  *   scale    multiplies q.k (1/sqrt(D) in the reference)
  *   max_context   upper bound of input_pos + 1, fixes the launch grid
  *   split_tokens  tokens per split, a multiple of 64 (0 = library default)
@@ -158,7 +163,7 @@ int fp_paged_decode(const void* q, int64_t q_stride_b, int64_t q_stride_h,
                     const int64_t* batch_idx,
                     const void* input_pos, int pos_index_type,
                     void* out, int64_t out_stride_b, int64_t out_stride_h,
-                    float* lse,
+                    float* lse, const float* sinks,
                     void* workspace, int64_t workspace_bytes,
                     int32_t B, int32_t Hq, int32_t Hc, int32_t D,
                     int32_t page_size, int32_t n_pages, int32_t max_batch,
@@ -183,7 +188,7 @@ int fp_paged_decode_partial(const void* q, int64_t q_stride_b, int64_t q_stride_
                             const int64_t* batch_idx,
                             const void* input_pos, int pos_index_type,
                             void* out, int64_t out_stride_b, int64_t out_stride_h,
-                            float* lse,
+                            float* lse, const float* sinks,
                             void* workspace, int64_t workspace_bytes,
                             int32_t B, int32_t Hq, int32_t Hc, int32_t D,
                             int32_t page_size, int32_t n_pages, int32_t max_batch,
@@ -196,7 +201,7 @@ int fp_paged_decode_merge(const void* q, int64_t q_stride_b, int64_t q_stride_h,
                           const int64_t* batch_idx,
                           const void* input_pos, int pos_index_type,
                           void* out, int64_t out_stride_b, int64_t out_stride_h,
-                          float* lse,
+                          float* lse, const float* sinks,
                           void* workspace, int64_t workspace_bytes,
                           int32_t B, int32_t Hq, int32_t Hc, int32_t D,
                           int32_t page_size, int32_t n_pages, int32_t max_batch,
@@ -224,7 +229,7 @@ int fp_paged_decode_append(const void* k_new, const void* v_new,
                            const int64_t* batch_idx,
                            const void* input_pos, int pos_index_type,
                            void* out, int64_t out_stride_b, int64_t out_stride_h,
-                           float* lse,
+                           float* lse, const float* sinks,
                            void* workspace, int64_t workspace_bytes,
                            int32_t B, int32_t Hq, int32_t Hc, int32_t D,
                            int32_t page_size, int32_t n_pages, int32_t max_batch,
@@ -259,13 +264,14 @@ int fp_hybrid_row_limits(const int64_t* input_ids, int32_t L,
  *              (row position + 1 for a causal row, the end of the image span inside one);
  *              every such key must already be in the pages
  *   out        [Lq, Hq, D] view, strides (row, head); lse [Hq, Lq] float32
+ *   sinks      NULL, or [Hq] float32 attention-sink logits, as in fp_paged_decode
  */
 int fp_paged_prefill(const void* q, int64_t q_stride_row, int64_t q_stride_h,
                      const void* pool_k, const void* pool_v,
                      const int64_t* page_table, int64_t pt_row_stride,
                      const int64_t* batch_idx, const int32_t* row_limit,
                      void* out, int64_t out_stride_row, int64_t out_stride_h,
-                     float* lse,
+                     float* lse, const float* sinks,
                      int32_t Lq, int32_t Hq, int32_t Hc, int32_t D,
                      int32_t page_size, int32_t n_pages, int32_t max_batch,
                      int64_t n_slots, float scale, int dtype,

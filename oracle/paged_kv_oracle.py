@@ -27,6 +27,9 @@ How each function is pinned (tests/test_oracle_*.py):
   decode_attention, prefill_attention   scipy logsumexp / torch SDPA (library
                           routines), L=1 closed form, equal-keys -> mean(V),
                           page-permutation invariance
+  round_to_dtype          torch's own casts (library routine), ties and specials
+  sink_gate               torch.sigmoid (library routine); closed forms: sink -> -inf
+                          leaves out unchanged, sink == lse halves it, lse = -inf zeroes it
 The reference holds no tests, golden vectors or fixtures for this path, so
 those mathematical pins are all there is; none of the functions is unpinned.
 """
@@ -435,3 +438,38 @@ def prefill_attention_paged(q, pool_k, pool_v, page_table, batch_idx, input_pos,
             s = (K[:n] @ q[0, h, r]) * scale
             out[0, h, r], lse[0, h, r] = _softmax_av(s, V[:n])
     return out, lse
+
+
+# --------------------------------------------------------------------------
+# post-attention sink gate
+# --------------------------------------------------------------------------
+def round_to_dtype(x, dtype: str):
+    """Value of float32 `x` after a round-to-nearest-even cast to `dtype` ("f32", "bf16", "f16") and back."""
+    x = np.asarray(x, dtype=np.float32)
+    if dtype == "f32":
+        return x.copy()
+    if dtype == "f16":
+        with np.errstate(over="ignore"):
+            return x.astype(np.float16).astype(np.float32)
+    if dtype == "bf16":
+        flat = np.ascontiguousarray(x).reshape(-1)
+        bits = flat.view(np.uint32).astype(np.uint64)
+        rounded = ((bits + 0x7FFF + ((bits >> 16) & 1)) & 0xFFFF0000).astype(np.uint32)
+        out = rounded.view(np.float32).copy()
+        out[np.isnan(flat)] = np.nan
+        return out.reshape(x.shape)
+    raise ValueError(dtype)
+
+
+def sink_gate(out, lse, sinks, dtype: str):
+    """Attention._post_attention up to the transpose (model.py:122-126).
+
+    out [B, H, S, D] attention output as values of the model dtype, lse [B, H, S] float32,
+    sinks [H].  `sink_scale = sigmoid(lse - sinks.view(1, -1, 1))` in float32 (:124-125);
+    `(out * sink_scale.unsqueeze(-1)).to(out.dtype)` (:126): float32 product, rounded to `dtype`."""
+    out = round_to_dtype(out, dtype)
+    lse = np.asarray(lse, dtype=np.float32)
+    sinks = np.asarray(sinks, dtype=np.float32).reshape(1, -1, 1)
+    with np.errstate(over="ignore"):
+        scale = (1.0 / (1.0 + np.exp(-(lse - sinks).astype(np.float64)))).astype(np.float32)
+    return round_to_dtype(out * scale[..., None], dtype)
