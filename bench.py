@@ -379,7 +379,32 @@ def append_gather_rates(steps: int = 20, T: int = 32768, H: int = 16, D: int = 1
     e = 2
     bytes_a = 2 * T * (2 * H * D * e) + 8 * T
     bytes_g = 2 * T * (H * D * e)
+
+    # QK norm + rotary embedding + insert in one launch (reference model.py:110-119 + the append):
+    # the qkv projection output of the same step, 16 query heads / 8 kv heads, expanded to the 16 cached heads
+    Hkv = H // 2
+    qkv = torch.randn((1, T, (H + 2 * Hkv) * D), device=dev, dtype=dtype)
+    xq, xk, xv = qkv.split([H * D, Hkv * D, Hkv * D], dim=-1)
+    xq, xk, xv = xq.view(1, T, H, D), xk.view(1, T, Hkv, D), xv.view(1, T, Hkv, D)
+    ang = torch.rand((1, T, D // 4), device=dev)
+    f1 = torch.polar(torch.ones_like(ang), ang)
+    ang2 = torch.rand((1, T, H, D // 4), device=dev)
+    f2 = torch.polar(torch.ones_like(ang2), ang2)
+    q_out = torch.empty((1, H, T, D), dtype=dtype, device=dev)
+
+    def do_rope():
+        ops.qkv_norm_rope_append(xq, xk, xv, f1, f2, pk, pv, cache.page_table, flat_b, pos.reshape(T), P,
+                                 clamp_negative=False, q_out=q_out)
+
+    for _ in range(3):
+        do_rope()
+    ms_r = event_ms(do_rope, steps)
+    # read q, k, v rows and both angle tables once, write q and the expanded K and V rows, token indices
+    bytes_r = (T * (H + 2 * Hkv) * D * e + T * (D // 4) * 8 + T * H * (D // 4) * 8
+               + T * H * D * e + 2 * T * H * D * e + 16 * T)
     return {"tokens": T, "heads": H, "head_dim": D,
+            "qkv_norm_rope_append_ms": ms_r, "qkv_norm_rope_append_gbps": bytes_r / (ms_r * 1e-3) / 1e9,
+            "qkv_norm_rope_append_frac_of_peak": bytes_r / (ms_r * 1e-3) / 1e9 / HBM_PEAK_GBPS,
             "kv_append_ms": ms_a, "kv_append_gbps": bytes_a / (ms_a * 1e-3) / 1e9,
             "kv_append_frac_of_peak": bytes_a / (ms_a * 1e-3) / 1e9 / HBM_PEAK_GBPS,
             "kv_gather_ms": ms_g, "kv_gather_gbps": bytes_g / (ms_g * 1e-3) / 1e9,

@@ -49,6 +49,12 @@ SIGNATURES = {
     "fp_paged_decode_partial": None,  # same signature as fp_paged_decode, filled in below
     "fp_paged_decode_merge": None,
     "fp_paged_decode_append": None,  # two row pointers and four strides in front of the same list
+    "fp_qkv_norm_rope_append": (c_int, [
+        c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+        c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p,
+        c_void_p, c_int64, c_void_p, c_void_p, c_int,
+        c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
+        c_int64, c_float, c_int, c_int, c_void_p]),
     "fp_hybrid_row_limits": (c_int, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_void_p]),
     "fp_paged_prefill": (c_int, [
         c_void_p, c_int64, c_int64, c_void_p, c_void_p,

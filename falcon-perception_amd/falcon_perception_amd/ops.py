@@ -51,6 +51,66 @@ def kv_append(pool_k: Tensor, pool_v: Tensor, k: Tensor, v: Tensor, page_table: 
     N.check(rc, "fp_kv_append")
 
 
+def qkv_norm_rope_append(xq: Tensor, xk: Tensor, xv: Tensor, freqs_cis: Tensor, freqs_cis_2d: Tensor | None,
+                         pool_k: Tensor, pool_v: Tensor, page_table: Tensor, batch_idx: Tensor, input_pos: Tensor,
+                         page_size: int, *, eps: float | None = None, clamp_negative: bool = True,
+                         q_out: Tensor | None = None) -> Tensor:
+    """RMS norm of q and k, head repeat, 3D rotary embedding and the cache insert in one launch
+    (reference `model.py:110-119` + `paged_attention.py:184-232, 364-393`).
+
+    xq [B, S, Hq, D], xk / xv [B, S, Hkv, D] (views of the qkv projection are fine); freqs_cis
+    [B, S, D/4] complex64, freqs_cis_2d None or [B, S, Hq, D/4] complex64; batch_idx and input_pos
+    one entry per token ([B*S] after flattening).  Returns the rotated q as [B, Hq, S, D]."""
+    N.require_cuda(xq, xk, xv, freqs_cis, freqs_cis_2d, pool_k, pool_v, page_table, batch_idx, input_pos, q_out)
+    B, S, Hq, D = xq.shape
+    Hkv = xk.shape[2]
+    if xk.shape != (B, S, Hkv, D) or xv.shape != xk.shape or xk.dtype != xq.dtype or xv.dtype != xq.dtype:
+        raise RuntimeError("xq / xk / xv shape or dtype mismatch")
+    if B > 1 and S > 1:
+        raise RuntimeError("one of batch and sequence must be 1 (decode [B, 1, ..] or packed prefill [1, L, ..])")
+    H_pool, n_slots, Dp = pool_k.shape
+    if Dp != D or pool_v.shape != pool_k.shape or pool_k.dtype != xq.dtype or pool_v.dtype != xq.dtype:
+        raise RuntimeError("pool shape or dtype mismatch")
+    T = B * S
+
+    def rows(x):  # [B, S, H, D] -> (tensor, token stride, head stride) with one stride for all tokens
+        if x.stride(3) != 1:
+            x = x.contiguous()
+        return x, (x.stride(1) if S > 1 else x.stride(0)), x.stride(2)
+
+    xq, qs_t, qs_h = rows(xq)
+    xk, ks_t, ks_h = rows(xk)
+    xv, vs_t, vs_h = rows(xv)
+    if freqs_cis.dtype != torch.complex64 or freqs_cis.shape != (B, S, D // 4):
+        raise RuntimeError("freqs_cis must be complex64 of shape [B, S, D/4]")
+    f1 = torch.view_as_real(freqs_cis.contiguous())
+    f2 = None
+    if freqs_cis_2d is not None:
+        if freqs_cis_2d.dtype != torch.complex64 or freqs_cis_2d.shape != (B, S, Hq, D // 4):
+            raise RuntimeError("freqs_cis_2d must be complex64 of shape [B, S, Hq, D/4]")
+        f2 = torch.view_as_real(freqs_cis_2d.contiguous())
+    batch_idx = batch_idx.reshape(-1).contiguous()
+    input_pos = input_pos.reshape(-1).contiguous()
+    if batch_idx.dtype != torch.int64 or batch_idx.shape[0] != T or input_pos.shape[0] != T:
+        raise RuntimeError("batch_idx (int64) and input_pos need one entry per token")
+    if q_out is None:
+        q_out = torch.empty((B, Hq, S, D), dtype=xq.dtype, device=xq.device)
+    if q_out.shape != (B, Hq, S, D) or q_out.stride(3) != 1:
+        raise RuntimeError("q_out must be [B, Hq, S, D] with dense rows")
+    if eps is None:
+        eps = torch.finfo(torch.float32).eps  # F.rms_norm(eps=None): epsilon of the fp32 computation type
+    rc = N.lib().fp_qkv_norm_rope_append(
+        xq.data_ptr(), xk.data_ptr(), xv.data_ptr(), qs_t, qs_h, ks_t, ks_h, vs_t, vs_h,
+        f1.data_ptr(), f2.data_ptr() if f2 is not None else None,
+        q_out.data_ptr(), q_out.stride(2) if S > 1 else q_out.stride(0), q_out.stride(1),
+        pool_k.data_ptr(), pool_v.data_ptr(), page_table.data_ptr(), page_table.stride(0),
+        batch_idx.data_ptr(), input_pos.data_ptr(), N.index_code(input_pos),
+        T, Hq, Hkv, H_pool, D, page_size, page_table.shape[1], page_table.shape[0], n_slots,
+        float(eps), N.dtype_code(xq.dtype), 1 if clamp_negative else 0, N.stream_ptr(xq.device))
+    N.check(rc, "fp_qkv_norm_rope_append")
+    return q_out
+
+
 def kv_gather(pool: Tensor, page_table: Tensor, batch_idx: Tensor, seq_lens: Tensor,
               page_size: int, max_len: int, out: Tensor | None = None) -> Tensor:
     """Dense logical view [B, H, max_len, D] of the cached rows of each sequence; zero tail."""

@@ -117,6 +117,33 @@ class PagedKVCache(KVCacheBase):
         self.last_prefill_step = StepMeta(layer_id, input_pos, batch_idx)
         return k_val, v_val
 
+    def insert_qkv_norm_rope(self, layer_id: int, xq: Tensor, xk: Tensor, xv: Tensor, freqs_cis: Tensor,
+                             freqs_cis_2d: Tensor | None = None, *, input_pos: Tensor, batch_idx: Tensor):
+        """`Attention._pre_attention` from the QK norm on (`model.py:110-119`) and `insert_kv`
+        (`model.py:150-153`) in one launch; not a method of the reference's class.
+
+        xq [B, S, n_heads, D], xk / xv [B, S, n_kv_heads, D]: the reshaped slices of the qkv
+        projection (`model.py:106-109`), views are fine.  Returns (q [B, n_heads, S, D], K, V) where
+        K, V are what `insert_kv` returns for a decode step (the layer's pool views); a prefill step
+        gets the pool views as well instead of the rotated fresh rows, which the paged prefill
+        attention does not read."""
+        decode = batch_idx.ndim == 1
+        assert batch_idx.ndim in [1, 2], "batch_idx must be 1D (decode) or 2D (prefill 1xL)"
+        B, S = xq.shape[0], xq.shape[1]
+        assert input_pos.shape == (B, S), "input_pos must be [B, S]"
+        if decode:
+            assert S == 1 and batch_idx.shape == (B,), "a decode step has one token per sequence"
+        else:
+            assert B == 1 and batch_idx.shape == (1, S), "a prefill step is one packed row"
+        q = ops.qkv_norm_rope_append(xq, xk, xv, freqs_cis, freqs_cis_2d, self.kv_cache[layer_id, 0, 0],
+                                     self.kv_cache[layer_id, 1, 0], self.page_table, batch_idx, input_pos,
+                                     self.page_size, clamp_negative=decode)
+        if decode:
+            self.last_decode_step = StepMeta(layer_id, input_pos, batch_idx)
+        else:
+            self.last_prefill_step = StepMeta(layer_id, input_pos, batch_idx)
+        return q, self.kv_cache[layer_id, 0], self.kv_cache[layer_id, 1]
+
     # --------------------------------------------------------------- allocator
     @property
     def num_free_pages(self) -> int:

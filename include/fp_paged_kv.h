@@ -238,6 +238,42 @@ int fp_paged_decode_append(const void* k_new, const void* v_new,
                            void* stream);
 
 /*
+ * Tail of Attention._pre_attention (model.py:110-119) and the cache insert that follows it
+ * (model.py:150-153 -> PagedKVCache.assign / assign_prefill_no_paging, paged_attention.py:184-232,
+ * 364-393) in one pass: RMS norm of q and k over head_dim (no weight), repeat of k and v to the
+ * cached head count, 3D rotary embedding (rope.py:88-108: 1D on the first half of head_dim with
+ * freqs_cis, "golden" 2D on the second half with per-head freqs_cis_2d when given), rotated q
+ * written in the caller's layout, K and V rows written to their pool slots.  Removes the
+ * repeat_kv / permute / .contiguous() copies and the separate append launch.
+ *
+ *   xq [T, Hq, D], xk, xv [T, Hkv, D] views with element strides (token, head): the slices of the
+ *              qkv projection, T = all tokens of the step (B for decode, packed length for prefill)
+ *   freqs_cis     [T, D/4, 2] float32 (cos, sin) = view_as_real of the reference's complex64 [.., D/4]
+ *   freqs_cis_2d  NULL or [T, Hq, D/4, 2] float32; needs H_pool == Hq
+ *   q_out      [T, Hq, D] view, element strides (token, head), e.g. those of a [B, H, S, D] tensor
+ *   pool_k/v   [H_pool, n_slots, D]; cached head h takes source head h / (H_pool / Hkv)
+ *   batch_idx, input_pos [T]: cache slot and position of every token
+ *   eps        added to mean(x^2); the reference passes eps=None, for which torch takes 2^-23
+ *              (the epsilon of the fp32 computation type) for every dtype
+ *   clamp_negative  as fp_kv_append (1 = decode semantics, 0 = prefill semantics)
+ * Rounding follows the reference: norm result rounded to dtype, rotation in fp32, rounded again.
+ */
+int fp_qkv_norm_rope_append(const void* xq, const void* xk, const void* xv,
+                            int64_t q_stride_t, int64_t q_stride_h,
+                            int64_t k_stride_t, int64_t k_stride_h,
+                            int64_t v_stride_t, int64_t v_stride_h,
+                            const float* freqs_cis, const float* freqs_cis_2d,
+                            void* q_out, int64_t qo_stride_t, int64_t qo_stride_h,
+                            void* pool_k, void* pool_v,
+                            const int64_t* page_table, int64_t pt_row_stride,
+                            const int64_t* batch_idx,
+                            const void* input_pos, int pos_index_type,
+                            int32_t T, int32_t Hq, int32_t Hkv, int32_t H_pool, int32_t D,
+                            int32_t page_size, int32_t n_pages, int32_t max_batch,
+                            int64_t n_slots, float eps, int dtype, int clamp_negative,
+                            void* stream);
+
+/*
  * Per-row key limits of the hybrid mask (bidirectional inside an image span,
  * causal elsewhere).  Replaces the compiled create_block_mask evaluation of
  * create_prefill_blockmask (paged_attention.py:343-362) with

@@ -27,6 +27,10 @@ How each function is pinned (tests/test_oracle_*.py):
   decode_attention, prefill_attention   scipy logsumexp / torch SDPA (library
                           routines), L=1 closed form, equal-keys -> mean(V),
                           page-permutation invariance
+  rms_norm_rows           torch F.rms_norm (library routine); unit rms of the result
+  rotary_3d               complex multiplication through torch.view_as_complex (library);
+                          zero angle = identity, quarter turn (a, b) -> (-b, a), pair norms kept
+  pre_attention_tail      composition of the two + numpy repeat against torch.repeat_interleave
   round_to_dtype          torch's own casts (library routine), ties and specials
   sink_gate               torch.sigmoid (library routine); closed forms: sink -> -inf
                           leaves out unchanged, sink == lse halves it, lse = -inf zeroes it
@@ -473,3 +477,54 @@ def sink_gate(out, lse, sinks, dtype: str):
     with np.errstate(over="ignore"):
         scale = (1.0 / (1.0 + np.exp(-(lse - sinks).astype(np.float64)))).astype(np.float32)
     return round_to_dtype(out * scale[..., None], dtype)
+
+
+# --------------------------------------------------------------------------
+# QK norm + 3D rotary embedding in front of the cache insert
+# --------------------------------------------------------------------------
+def rms_norm_rows(x, eps, dtype: str):
+    """F.rms_norm(x, (D,)) without weight (model.py:110-111): x * rsqrt(mean(x^2, -1) + eps) in
+    float32, returned as values of `dtype`.  The reference passes eps=None, for which torch takes the
+    machine epsilon of the float32 computation type also for bf16/f16 inputs (pinned against
+    torch.nn.functional.rms_norm: bit-identical with 2^-23, not with the epsilon of bf16)."""
+    x = np.asarray(x, dtype=np.float32)
+    ms = np.mean(x.astype(np.float64) ** 2, axis=-1, keepdims=True).astype(np.float32)
+    rstd = (1.0 / np.sqrt(ms.astype(np.float64) + eps)).astype(np.float32)
+    return round_to_dtype(x * rstd, dtype)
+
+
+def rotary_3d(x, freqs_cis, freqs_cis_2d, dtype: str):
+    """apply_3d_rotary_emb for one tensor (rope.py:88-108).  x [B, S, H, D] values of `dtype`;
+    freqs_cis complex [B, S, D/4] (rope.py:31-46: pairs (2i, 2i+1) of the first half times
+    freqs_cis[b, s, i], broadcast over heads); freqs_cis_2d complex [B, S, H, D/4] or None
+    (rope.py:71-86: even/odd elements of the second half rotated by the per-head angle)."""
+    x = np.asarray(x, dtype=np.float32)
+    D = x.shape[-1]
+    half = D // 2
+    out = x.copy()
+
+    def rotate(part, cis):  # part [..., half] float32, cis complex broadcastable to [..., half/2]
+        re, im = part[..., 0::2], part[..., 1::2]
+        c = np.real(cis).astype(np.float32)
+        s_ = np.imag(cis).astype(np.float32)
+        res = np.empty_like(part)
+        res[..., 0::2] = re * c - im * s_
+        res[..., 1::2] = re * s_ + im * c
+        return res
+
+    out[..., :half] = rotate(x[..., :half], np.asarray(freqs_cis)[:, :, None, :])
+    if freqs_cis_2d is not None:
+        out[..., half:] = rotate(x[..., half:], np.asarray(freqs_cis_2d))
+    return round_to_dtype(out, dtype)
+
+
+def pre_attention_tail(xq, xk, xv, freqs_cis, freqs_cis_2d, n_rep: int, dtype: str, eps: float):
+    """model.py:110-119: QK norm, repeat_kv (model.py:74-83, repeat_interleave along heads),
+    3D rotary embedding, permute to [B, H, S, D].  Returns (q, k, v) as float32 values of `dtype`."""
+    q = rms_norm_rows(xq, eps, dtype)
+    k = rms_norm_rows(xk, eps, dtype)
+    k = np.repeat(k, n_rep, axis=2)
+    v = np.repeat(round_to_dtype(xv, dtype), n_rep, axis=2)
+    q = rotary_3d(q, freqs_cis, freqs_cis_2d, dtype)
+    k = rotary_3d(k, freqs_cis, freqs_cis_2d, dtype)
+    return q.transpose(0, 2, 1, 3), k.transpose(0, 2, 1, 3), v.transpose(0, 2, 1, 3)
