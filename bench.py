@@ -162,7 +162,10 @@ def make_decode_case(name: str, device="cuda", hbm_budget_gb: float | None = Non
         n_pages = max(need_pages, int(budget // page_bytes))
     assert need_pages <= n_pages, f"{name}: {need_pages} pages needed, pool has {n_pages}"
     c["n_pages"] = n_pages
-    cache = PagedKVCache(n_pages, P, B + 1, c["Hc"], c["D"], 1, dtype, device=device)
+    # a pool of several hundred thousand pages gets a sparse page table (columns = blocks of the longest
+    # sequence): the reference's dense [B + 1, n_pages] int64 pair would be 1.4 GB at cfg5
+    cols = math.ceil((max(lens) + 1) / P) if DECODE_WORKLOADS[name]["n_pages"] is None else None
+    cache = PagedKVCache(n_pages, P, B + 1, c["Hc"], c["D"], 1, dtype, device=device, max_blocks_per_seq=cols)
     perm = (torch.randperm(n_pages - 1, generator=gen) + 1).tolist()
     cache.free_pages = perm
     slots = []

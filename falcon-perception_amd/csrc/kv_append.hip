@@ -120,8 +120,8 @@ extern "C" int fp_kv_append(void* pool_k, void* pool_v, const void* k, const voi
   if (H > 65535) return fp::fail(FP_ERR_UNSUPPORTED, "fp_kv_append: H=%d exceeds 65535", H);
   if (static_cast<int64_t>(T) * S > INT32_MAX)
     return fp::fail(FP_ERR_UNSUPPORTED, "fp_kv_append: more than 2^31-1 tokens");
-  if (n_slots < static_cast<int64_t>(n_pages) * page_size)
-    return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_kv_append: n_slots smaller than n_pages * page_size");
+  if (n_slots < page_size)
+    return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_kv_append: n_slots smaller than one page");
   if (pos_index_type != FP_INDEX_I32 && pos_index_type != FP_INDEX_I64)
     return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_kv_append: bad pos_index_type");
   if (T == 0) return FP_OK;

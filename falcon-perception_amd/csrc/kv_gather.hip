@@ -120,8 +120,8 @@ extern "C" int fp_kv_gather(const void* pool, void* out, int64_t out_stride_b, i
   if (B < 0 || H <= 0 || max_len < 0 || D <= 0 || page_size <= 0 || n_pages <= 0 || max_batch <= 0 || n_slots <= 0)
     return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_kv_gather: non-positive dimension");
   if (H > 65535 || B > 65535) return fp::fail(FP_ERR_UNSUPPORTED, "fp_kv_gather: B or H exceeds 65535");
-  if (n_slots < static_cast<int64_t>(n_pages) * page_size)
-    return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_kv_gather: n_slots smaller than n_pages * page_size");
+  if (n_slots < page_size)
+    return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_kv_gather: n_slots smaller than one page");
   if (len_index_type != FP_INDEX_I32 && len_index_type != FP_INDEX_I64)
     return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_kv_gather: bad len_index_type");
   if (B == 0 || max_len == 0) return FP_OK;

@@ -317,7 +317,7 @@ __global__ __launch_bounds__(kThreads) void paged_decode_kernel(const DecodeArgs
     for (int i = tid; i < nblk; i += kThreads) {
       int64_t page = 0;
       if (blk0 + i < a.n_pages) page = a.page_table[trow * a.pt_row_stride + blk0 + i];
-      if (page < 0 || page >= a.n_pages) page = 0;
+      if (page < 0 || page >= a.n_slots / a.pd.page_size) page = 0;  // not a page of the pool
       s_pages[i] = static_cast<int>(page);
     }
   }
@@ -587,8 +587,8 @@ int decode_entry(int phases, const NewRows* fresh, const void* q, int64_t q_stri
       n_slots <= 0 || max_context < 0 || split_tokens < 0)
     return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: bad dimension");
   if (Hq % Hc) return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: Hq=%d not a multiple of Hc=%d", Hq, Hc);
-  if (n_slots < static_cast<int64_t>(n_pages) * page_size)
-    return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: n_slots smaller than n_pages * page_size");
+  if (n_slots < page_size)
+    return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: n_slots smaller than one page");
   if (max_context > static_cast<int64_t>(n_pages) * page_size)
     return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: max_context exceeds the page table width");
   if (pos_index_type != FP_INDEX_I32 && pos_index_type != FP_INDEX_I64)

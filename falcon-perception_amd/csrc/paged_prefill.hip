@@ -303,13 +303,14 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
         page_next[i] = pt_row[(kpos < kv_max && blkid < a.n_pages) ? blkid : 0];
       }
     };
+    const int64_t pool_pages = a.n_slots / a.pd.page_size;
     auto resolve = [&](int kt) {  // page_next holds the ids of tile kt
 #pragma unroll
       for (int i = 0; i < NI; ++i) {
         const int kpos = kt * kTileN + i * kWaves * RPI + st_row0;
         int blkid, off;
         key_block(kpos, blkid, off);
-        const bool ok = kpos < kv_max && blkid < a.n_pages && page_next[i] >= 0 && page_next[i] < a.n_pages;
+        const bool ok = kpos < kv_max && blkid < a.n_pages && page_next[i] >= 0 && page_next[i] < pool_pages;
         const int slot = ok ? static_cast<int>(page_next[i]) * a.pd.page_size + off : 0;
         rowbyte[i] = static_cast<int64_t>(slot) * ROWB;
       }
@@ -542,8 +543,8 @@ extern "C" int fp_paged_prefill(const void* q, int64_t q_stride_row, int64_t q_s
   if (Lq < 0 || Hq <= 0 || Hc <= 0 || page_size <= 0 || n_pages <= 0 || max_batch <= 0 || n_slots <= 0)
     return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_prefill: bad dimension");
   if (Hq % Hc) return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_prefill: Hq=%d not a multiple of Hc=%d", Hq, Hc);
-  if (n_slots < static_cast<int64_t>(n_pages) * page_size)
-    return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_prefill: n_slots smaller than n_pages * page_size");
+  if (n_slots < page_size)
+    return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_prefill: n_slots smaller than one page");
   if (Hc > 65535) return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill: Hc exceeds 65535");
   if (n_slots > INT32_MAX) return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill: more than 2^31-1 slots per head");
   if (Lq == 0) return FP_OK;

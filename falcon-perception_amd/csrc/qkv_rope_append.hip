@@ -246,8 +246,8 @@ extern "C" int fp_qkv_norm_rope_append(const void* xq, const void* xk, const voi
   const int tpr = D / epv;
   if (D % (2 * epv) || (tpr & (tpr - 1)) || tpr > 64)
     return fp::fail(FP_ERR_UNSUPPORTED, "fp_qkv_norm_rope_append: head_dim %d for %d-byte elements", D, eb);
-  if (n_slots < static_cast<int64_t>(n_pages) * page_size)
-    return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_qkv_norm_rope_append: n_slots smaller than n_pages * page_size");
+  if (n_slots < page_size)
+    return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_qkv_norm_rope_append: n_slots smaller than one page");
   if (pos_index_type != FP_INDEX_I32 && pos_index_type != FP_INDEX_I64)
     return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_qkv_norm_rope_append: bad pos_index_type");
   if (T == 0) return FP_OK;

@@ -15,7 +15,7 @@ import torch
 _LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib")
 LIB_PATH = os.path.join(_LIB_DIR, "libfp_paged_kv.so")
 
-FP_ABI_VERSION = 1
+FP_ABI_VERSION = 2
 FP_DTYPE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
 FP_INDEX = {torch.int32: 0, torch.int64: 1}
 

@@ -65,7 +65,7 @@ class PagedDecodeMask:
     @property
     def max_context(self) -> int:
         """Upper bound of the logical context length (KV length of the logical mask)."""
-        return min(int(self.logical.seq_lengths[1]), self.cache.n_pages * self.cache.page_size)
+        return min(int(self.logical.seq_lengths[1]), self.cache.table_cols * self.cache.page_size)
 
     def _converted(self, name: str) -> Tensor | None:
         if name not in self._physical:

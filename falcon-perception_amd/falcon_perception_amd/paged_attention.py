@@ -43,19 +43,32 @@ class PagedKVCache(KVCacheBase):
       physical_to_logical [max_batch, n_pages] int64 inverse map (:70)
       page_table_cpu, capacity, free_pages, free_batch_idx   host mirrors (:60-67);
                           page 0 and batch slot 0 are reserved and never handed out
+
+    `max_blocks_per_seq` (not an argument of the reference's class) makes the tables sparse:
+    page_table becomes [max_batch, max_blocks_per_seq] and the inverse table is not kept.  The
+    reference's dense [max_batch, n_pages] int64 pair grows with pool size times batch size
+    (1.4 GB for 257 slots over a 343 k-page pool); the kernels only ever read
+    page_table[slot, block], so the narrow table serves them unchanged.  What needs the inverse
+    table (`get_mask_mod`, the element mask of the reference's flex kernels) is then unavailable.
     """
 
     def __init__(self, n_pages: int, page_size: int, max_batch_size: int, n_heads: int, head_dim: int,
-                 num_layers: int, dtype: torch.dtype, device: str | torch.device = "cuda"):
+                 num_layers: int, dtype: torch.dtype, device: str | torch.device = "cuda",
+                 max_blocks_per_seq: int | None = None):
         self.n_pages = n_pages
         self.page_size = page_size
         self.max_batch_size = max_batch_size
         self.dtype = dtype
         self.device = device
 
-        self.page_table = torch.full((max_batch_size, n_pages), -1, dtype=torch.int64, device=device)
+        self.table_cols = n_pages if max_blocks_per_seq is None else int(max_blocks_per_seq)
+        if not 0 < self.table_cols <= n_pages:
+            raise ValueError("max_blocks_per_seq must be between 1 and n_pages")
+        self.page_table = torch.full((max_batch_size, self.table_cols), -1, dtype=torch.int64, device=device)
         self.page_table[0].zero_()
-        self.physical_to_logical = torch.full((max_batch_size, n_pages), -1, dtype=torch.int64, device=device)
+        self.physical_to_logical = None
+        if max_blocks_per_seq is None:
+            self.physical_to_logical = torch.full((max_batch_size, n_pages), -1, dtype=torch.int64, device=device)
         self.page_table_cpu: list[list[int]] = [[] for _ in range(max_batch_size)]
         self.capacity: list[int] = [0] * max_batch_size
         self.free_pages: list[int] = list(range(n_pages - 1, 0, -1))
@@ -159,7 +172,8 @@ class PagedKVCache(KVCacheBase):
         """Take a free batch slot and clear its table rows (:102-109)."""
         slot = self.free_batch_idx.pop()
         self.capacity[slot] = 0
-        self.physical_to_logical[slot].fill_(-1)
+        if self.physical_to_logical is not None:
+            self.physical_to_logical[slot].fill_(-1)
         self.page_table[slot].fill_(-1)
         return slot
 
@@ -174,6 +188,13 @@ class PagedKVCache(KVCacheBase):
             return True
         n_new = _cdiv(seq_len - have, self.page_size)
         fits = bool(n_new <= self.num_free_pages)
+        if have // self.page_size + n_new > self.table_cols:  # only a sparse table can be narrower than the pool
+            if dry_run:
+                return False
+            raise RuntimeError(
+                f"Cannot reserve a sequence of length {seq_len} in batch {batch_idx_int}: "
+                f"the page table holds {self.table_cols} blocks of {self.page_size} tokens per sequence."
+            )
         if dry_run:
             return fits
         if not fits:
@@ -188,7 +209,8 @@ class PagedKVCache(KVCacheBase):
         pages_dev = torch.tensor(pages, device=self.device)
         row = batch_idx_int  # the tensor argument of the reference names the same slot
         self.page_table[row, first:first + n_new] = pages_dev
-        self.physical_to_logical[row, pages_dev] = torch.arange(first, first + n_new, device=self.device)
+        if self.physical_to_logical is not None:
+            self.physical_to_logical[row, pages_dev] = torch.arange(first, first + n_new, device=self.device)
         self.page_table_cpu[batch_idx_int] += pages
         self.capacity[batch_idx_int] = have + n_new * self.page_size
         return True
@@ -199,7 +221,8 @@ class PagedKVCache(KVCacheBase):
         self.free_pages.extend(reversed(self.page_table_cpu[batch_idx]))
         self.page_table_cpu[batch_idx] = []
         self.page_table[batch_idx].fill_(-1)
-        self.physical_to_logical[batch_idx].fill_(-1)
+        if self.physical_to_logical is not None:
+            self.physical_to_logical[batch_idx].fill_(-1)
         self.capacity[batch_idx] = 0
 
     # ------------------------------------------------------------------- masks
@@ -224,6 +247,8 @@ class PagedKVCache(KVCacheBase):
 
     def get_logical_kv_idx(self, physical_batch_idx: Tensor, physical_kv_idx: Tensor, batch_idx: Tensor):
         """Physical slot -> (mapped?, logical position) for one batch row (:303-311)."""
+        if self.physical_to_logical is None:
+            raise RuntimeError("this cache was built with max_blocks_per_seq: it keeps no physical_to_logical table")
         slot_row = batch_idx[physical_batch_idx]
         block = self.physical_to_logical[slot_row, physical_kv_idx // self.page_size]
         logical = block * self.page_size + physical_kv_idx % self.page_size

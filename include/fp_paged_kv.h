@@ -19,6 +19,12 @@
  *  - Indices that fall outside the tables or the pool (a slot < 0 or >= n_slots,
  *    a batch index >= max_batch, a block id >= n_pages) are skipped on the
  *    device instead of faulting; the reference raises an index error there.
+ *  - `n_pages` is the number of COLUMNS of page_table, i.e. the logical blocks one
+ *    sequence can map.  The reference's table has one column per pool page
+ *    (paged_attention.py:58); a narrower table [max_batch, max blocks per sequence]
+ *    works the same and is what a pool of several hundred thousand pages needs.
+ *    The pool's own page count is n_slots / page_size; page ids outside it count as
+ *    unmapped.
  */
 #ifndef FP_PAGED_KV_H
 #define FP_PAGED_KV_H
@@ -29,7 +35,7 @@
 extern "C" {
 #endif
 
-#define FP_ABI_VERSION 1
+#define FP_ABI_VERSION 2
 
 /* element types of pool / q / k / v */
 #define FP_DTYPE_F32 0

@@ -33,9 +33,11 @@ def randn(gen, shape, dtype):
 class PagedState:
     """A PagedKVCache on the GPU plus an oracle mirror of its tables and pool."""
 
-    def __init__(self, seed, *, n_pages, page_size, max_batch, Hc, D, dtype, n_layers=1, shuffle=True):
+    def __init__(self, seed, *, n_pages, page_size, max_batch, Hc, D, dtype, n_layers=1, shuffle=True,
+                 max_blocks_per_seq=None):
         self.gen = torch.Generator().manual_seed(seed)
-        self.cache = PagedKVCache(n_pages, page_size, max_batch, Hc, D, n_layers, dtype, device=DEV)
+        self.cache = PagedKVCache(n_pages, page_size, max_batch, Hc, D, n_layers, dtype, device=DEV,
+                                  max_blocks_per_seq=max_blocks_per_seq)
         self.mirror = O.PagedAllocator(n_pages, page_size, max_batch)
         if shuffle:
             perm = (torch.randperm(n_pages - 1, generator=self.gen) + 1).tolist()

@@ -214,3 +214,29 @@ def test_install_serves_the_reference_module_names():
                 sys.modules.pop(k, None)
             else:
                 sys.modules[k] = v
+
+
+def test_sparse_page_table_allocator():
+    """max_blocks_per_seq: same allocator decisions as the dense table (free lists, capacities, the
+    mapped prefix of every row), a narrower table, no inverse table, and a per-sequence length limit."""
+    dense = PagedKVCache(40, 4, 5, 1, 4, 1, torch.float32, device="cpu")
+    sparse = PagedKVCache(40, 4, 5, 1, 4, 1, torch.float32, device="cpu", max_blocks_per_seq=6)
+    assert sparse.page_table.shape == (5, 6) and sparse.physical_to_logical is None
+    assert sparse.page_table[0].tolist() == [0] * 6  # the reserved row still points at page 0
+    for c in (dense, sparse):
+        a, b = c.allocate(), c.allocate()
+        c.reserve(a, None, 9)
+        c.reserve(b, None, 24)
+        c.reserve(a, None, 13)
+        c.erase(b)
+        b2 = c.allocate()
+        c.reserve(b2, None, 5)
+    assert sparse.free_pages == dense.free_pages and sparse.capacity == dense.capacity
+    assert sparse.page_table_cpu == dense.page_table_cpu
+    assert sparse.page_table.tolist() == dense.page_table[:, :6].tolist()
+    assert int(sparse.page_table.max()) >= 6  # page ids are not bounded by the table width
+    assert sparse.can_reserve(24, 1) is True and sparse.can_reserve(25, 1) is False and dense.can_reserve(25, 1) is True
+    with pytest.raises(RuntimeError, match="6 blocks"):
+        sparse.reserve(1, None, 25)
+    with pytest.raises(ValueError):
+        PagedKVCache(8, 4, 2, 1, 4, 1, torch.float32, device="cpu", max_blocks_per_seq=9)
