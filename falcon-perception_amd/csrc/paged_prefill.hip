@@ -537,8 +537,8 @@ extern "C" int fp_paged_prefill(const void* q, int64_t q_stride_row, int64_t q_s
                                 int32_t Lq, int32_t Hq,
                                 int32_t Hc, int32_t D, int32_t page_size, int32_t n_pages, int32_t max_batch,
                                 int64_t n_slots, float scale, int dtype, void* stream) {
-  if (dtype != FP_DTYPE_BF16 && dtype != FP_DTYPE_F16)
-    return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill: dtype %d (supported: bf16, f16)", dtype);
+  if (dtype != FP_DTYPE_BF16 && dtype != FP_DTYPE_F16 && dtype != FP_DTYPE_F32)
+    return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill: unknown dtype %d", dtype);
   if (D != 64 && D != 128) return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill: head_dim %d (supported: 64, 128)", D);
   if (Lq < 0 || Hq <= 0 || Hc <= 0 || page_size <= 0 || n_pages <= 0 || max_batch <= 0 || n_slots <= 0)
     return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_prefill: bad dimension");
@@ -550,11 +550,21 @@ extern "C" int fp_paged_prefill(const void* q, int64_t q_stride_row, int64_t q_s
   if (Lq == 0) return FP_OK;
   if (!q || !pool_k || !pool_v || !page_table || !batch_idx || !row_limit || !out || !lse)
     return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_prefill: null pointer");
+  if (dtype == FP_DTYPE_F32) {
+    // no fp32 MFMA kernel: the rows go through the single-query kernel, one row per workgroup
+    if (!fp::aligned(q, 16) || !fp::aligned(pool_k, 16) || !fp::aligned(pool_v, 16) || !fp::aligned(out, 4) ||
+        (q_stride_row * 4) % 16 || (q_stride_h * 4) % 16)
+      return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_prefill: q rows must be 16-byte aligned");
+    const int rc32 = fp::prefill_rows_f32(q, q_stride_row, q_stride_h, pool_k, pool_v, page_table, pt_row_stride, batch_idx,
+                                          row_limit, out, out_stride_row, out_stride_h, lse, sinks, Lq, Hq, Hc, D, page_size,
+                                          n_pages, max_batch, n_slots, scale, static_cast<hipStream_t>(stream));
+    if (rc32 != FP_OK) return rc32;
+    return fp::check_launch("fp_paged_prefill");
+  }
   if (!fp::aligned(q, 16) || !fp::aligned(pool_k, 16) || !fp::aligned(pool_v, 16) || !fp::aligned(out, 8) ||
       (q_stride_row * 2) % 16 || (q_stride_h * 2) % 16 || (out_stride_row * 2) % 8 || (out_stride_h * 2) % 8)
     return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_prefill: q rows must be 16-byte and out rows 8-byte aligned");
   if ((static_cast<int64_t>(Lq) + 31) / 32 > 65535) return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill: too many query rows");
-
   PrefillArgs a{static_cast<const char*>(q), q_stride_row * 2, q_stride_h * 2,
                 static_cast<const char*>(pool_k), static_cast<const char*>(pool_v),
                 page_table, pt_row_stride, batch_idx, row_limit,

@@ -14,7 +14,7 @@ from tests.test_oracle_masks import EOI, IMG, PAD, SOI, TXT, packed_case
 
 pytestmark = pytest.mark.gpu
 
-TOL = {torch.bfloat16: (2e-2, 1e-2), torch.float16: (4e-3, 4e-3)}
+TOL = {torch.bfloat16: (2e-2, 1e-2), torch.float16: (4e-3, 4e-3), torch.float32: (2e-5, 2e-5)}
 
 
 def assert_close(out, lse, eo, el, dtype, rows=None):
@@ -65,7 +65,7 @@ def repack(layout, pad_to):
     return np.array(ids), np.array(bidx), np.array(pos)
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=str)
 @pytest.mark.parametrize("D,G", [(128, 1), (128, 2), (64, 4)])
 def test_whole_sequence_prefill_matches_the_reference_semantics(dtype, D, G):
     """The reference's own prefill (packed sequences, each padded to 128): attention over the packed
@@ -162,3 +162,24 @@ def test_cfg3_chunked_prefill_shape():
         eo, el = O.prefill_attention_paged(f64(case.q[:, :, rows]), pk, pv, case.page_table.cpu().numpy(),
                                            bidx[rows], None, lim[rows], case.page_size)
         assert_close(out[:, :, rows], lse[:, :, rows], eo, el, torch.bfloat16)
+
+
+def test_fp32_rows_over_a_context_longer_than_the_page_list():
+    """fp32 (the reference's default dtype) has no MFMA kernel: rows go through the single-query kernel,
+    whose LDS page list holds 512 pages per round.  Limits on both sides of that boundary, page size 16."""
+    dtype, P, D = torch.float32, 16, 64
+    st = PagedState(9, n_pages=640, page_size=P, max_batch=3, Hc=1, D=D, dtype=dtype)
+    b = st.add_sequence(9000)
+    st.prefill_random()
+    lims = [0, 1, 8191, 8192, 8193, 9000, 16 * 512 + 16 * 3 + 5]
+    q = randn(st.gen, (1, 2, len(lims), D), dtype)
+    bidx = torch.full((len(lims),), b, dtype=torch.int64)
+    bidx[1] = 0  # a padding row: out 0, lse -inf whatever its limit
+    lim = torch.tensor(lims, dtype=torch.int32)
+    pk, pv = st.pool_planes()
+    out, lse = ops.paged_prefill(q.to(DEV), pk, pv, st.cache.page_table, bidx.to(DEV), lim.to(DEV), P)
+    eo, el = O.prefill_attention_paged(f64(q), f64(pk), f64(pv), st.mirror.page_table, bidx.numpy(),
+                                       None, lim.numpy(), P)
+    assert_close(out, lse, eo, el, dtype)
+    assert not f64(out)[:, :, :2].any() and np.isneginf(f64(lse)[:, :, :2]).all()
+    assert lse.shape == (1, 2, len(lims))
