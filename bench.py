@@ -38,6 +38,9 @@ DECODE_WORKLOADS = {
     "cfg1": dict(seed=1, dtype="f32", B=4, Hq=8, Hc=8, D=64, P=64, n_pages=64, prefix=0, lo=64, hi=512),
     "cfg2": dict(seed=2, dtype="bf16", B=64, Hq=16, Hc=8, D=128, P=128, n_pages=4096, prefix=1024, lo=64, hi=3072),
     "cfg2x": dict(seed=2, dtype="bf16", B=64, Hq=16, Hc=16, D=128, P=128, n_pages=4096, prefix=1024, lo=64, hi=3072),
+    # the same expanded cache read as what it is: K per query head, V in groups of 2 identical copies
+    "cfg2xs": dict(seed=2, dtype="bf16", B=64, Hq=16, Hc=16, D=128, P=128, n_pages=4096, prefix=1024, lo=64, hi=3072,
+                   kv_rep=2),
     "cfg4d": dict(seed=4, dtype="bf16", B=32, Hq=16, Hc=8, D=128, P=64, n_pages=8192, prefix=0, lo=512, hi=8192),
     "cfg5": dict(seed=5, dtype="bf16", B=256, Hq=32, Hc=8, D=128, P=128, n_pages=None, prefix=4096, lo=256, hi=12288),
 }
@@ -96,7 +99,7 @@ class DecodeCase:
         return ops.paged_decode(self.q, self.pool_k, self.pool_v, self.cache.page_table, self.batch_idx,
                                 self.input_pos, self.page_size, self.max_context,
                                 split_tokens=self.split_tokens, workspace=self.workspace,
-                                out=self.out, lse=self.lse, phase=phase)
+                                out=self.out, lse=self.lse, phase=phase, kv_rep=self.cfg.get("kv_rep", 1))
 
     def run(self):
         self.append()
@@ -109,7 +112,8 @@ class DecodeCase:
         return ops.paged_decode(self.q, self.pool_k, self.pool_v, self.cache.page_table, self.batch_idx,
                                 self.input_pos, self.page_size, self.max_context,
                                 split_tokens=self.split_tokens, workspace=self.workspace,
-                                out=self.out, lse=self.lse, k_new=self.k_new, v_new=self.v_new)
+                                out=self.out, lse=self.lse, k_new=self.k_new, v_new=self.v_new,
+                                kv_rep=self.cfg.get("kv_rep", 1))
 
     def run_fused_gated(self):
         """run_fused plus the caller's post-attention sink gate (reference model.py:122-127) inside the
@@ -125,7 +129,7 @@ class DecodeCase:
                                 self.input_pos, self.page_size, self.max_context,
                                 split_tokens=self.split_tokens, workspace=self.workspace,
                                 out=out, lse=self.lse, k_new=self.k_new, v_new=self.v_new,
-                                sinks=self.extra["sinks"])
+                                sinks=self.extra["sinks"], kv_rep=self.cfg.get("kv_rep", 1))
 
     # ---- algorithmic traffic (bytes) --------------------------------------
     def bytes_append(self):
@@ -138,7 +142,9 @@ class DecodeCase:
         c = self.cfg
         e = self.q.element_size()
         ctx = [L + 1 for L in self.lens]  # the new token attends to itself
-        return (sum(ctx) * 2 * c["Hc"] * c["D"] * e + 2 * c["B"] * c["Hq"] * c["D"] * e + 4 * c["B"] * c["Hq"]
+        # K rows of every cached head, V rows of every DISTINCT cached head (identical copies count once)
+        heads_read = c["Hc"] + c["Hc"] // c.get("kv_rep", 1)
+        return (sum(ctx) * heads_read * c["D"] * e + 2 * c["B"] * c["Hq"] * c["D"] * e + 4 * c["B"] * c["Hq"]
                 + 8 * sum(math.ceil(x / c["P"]) for x in ctx))
 
 
@@ -184,7 +190,7 @@ def make_decode_case(name: str, device="cuda", hbm_budget_gb: float | None = Non
     max_context = min(n_pages * P, math.ceil((max(lens) + 1) / P) * P)
     case = DecodeCase(name, c, cache, lens, torch.tensor(slots, dtype=torch.int64, device=device),
                       torch.tensor(lens, dtype=torch.int32, device=device), q, k_new, v_new, max_context)
-    case.split_tokens = ops.decode_split_tokens(B, c["Hc"], max_context, P)
+    case.split_tokens = ops.decode_split_tokens(B, c["Hc"] // c.get("kv_rep", 1), max_context, P)
     need = ops.decode_workspace_bytes(B, c["Hq"], c["D"], max_context, case.split_tokens)
     case.workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=device)
     case.out = torch.empty_like(q)

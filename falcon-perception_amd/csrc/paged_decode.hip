@@ -202,8 +202,10 @@ __device__ __forceinline__ int split_part(int L, int split_tokens) {
 // One wavefront iteration: U row loads of K and V per lane are already in registers;
 // fold them into the lane group's online-softmax state.  kMasked: rows at or past
 // `t1` (only in the last iteration of a split) get a score of -inf.
-template <typename E, int TPR, int G, int U, int RPW, bool kMasked>
-__device__ __forceinline__ void fold_rows(const v4u (&kreg)[U], const v4u (&vreg)[U], const typename E::Q (&q)[G],
+// GK = 1: the G query heads share one K row; GK = G: every query head has its own K row (a cache
+// that stores one K head per query head) while V is still shared.
+template <typename E, int TPR, int G, int GK, int U, int RPW, bool kMasked>
+__device__ __forceinline__ void fold_rows(const v4u (&kreg)[GK][U], const v4u (&vreg)[U], const typename E::Q (&q)[G],
                                           float qscale, int row0, int t1, float (&m)[G], float (&l)[G],
                                           float (&acc)[G][E::kEpl]) {
   constexpr int EPL = E::kEpl;
@@ -211,7 +213,7 @@ __device__ __forceinline__ void fold_rows(const v4u (&kreg)[U], const v4u (&vreg
 #pragma unroll
   for (int u = 0; u < U; ++u) {
 #pragma unroll
-    for (int g = 0; g < G; ++g) s[g][u] = E::dot(q[g], kreg[u]);
+    for (int g = 0; g < G; ++g) s[g][u] = E::dot(q[g], kreg[GK == 1 ? 0 : g][u]);
   }
 #pragma unroll
   for (int g = 0; g < G; ++g) {
@@ -260,12 +262,20 @@ __device__ __forceinline__ void fold_rows(const v4u (&kreg)[U], const v4u (&vreg
 // a "sequence" of its own (grid y = row), input_pos holds the row's key limit (not limit - 1), rows
 // of cache slot 0 are padding, lse is [Hq, rows], and the one split of a row may span more pages
 // than the LDS page list holds, so the list is refilled every 512 pages.
-template <typename E, int D, int G, bool kDirect, bool kAligned, bool kRowMode = false>
+//
+// kPerHeadK serves a cache that holds one K head per QUERY head (the reference stores K and V
+// expanded to n_heads because the 2D rotary angles differ per head, model.py:112-114) whose V heads
+// are n_rep identical copies: a workgroup takes the G = n_rep query heads of one group, reads their G
+// K rows and ONE V row (the first copy), i.e. (G + 1) / 2G of the bytes an expanded read costs.
+constexpr int decode_loads_in_flight(int G, bool per_head_k) { return per_head_k && G >= 4 ? 4 : 8; }
+
+template <typename E, int D, int G, bool kDirect, bool kAligned, bool kRowMode = false, bool kPerHeadK = false>
 __global__ __launch_bounds__(kThreads) void paged_decode_kernel(const DecodeArgs a) {
   constexpr int EPL = E::kEpl;          // elements per lane
   constexpr int TPR = D / EPL;          // lanes per row
   constexpr int RPW = 64 / TPR;         // rows per wavefront load
-  constexpr int U = 8;                  // loads of K (and of V) in flight per lane
+  constexpr int GK = kPerHeadK ? G : 1; // K rows per token a workgroup reads
+  constexpr int U = decode_loads_in_flight(G, kPerHeadK);  // loads of K (per K head) and of V in flight per lane
   constexpr int CH = RPW * U;           // rows per wavefront iteration
   constexpr int ROWB = D * sizeof(typename E::type);
 
@@ -330,8 +340,11 @@ __global__ __launch_bounds__(kThreads) void paged_decode_kernel(const DecodeArgs
     for (int e = 0; e < EPL; ++e) acc[g][e] = 0.f;
   }
 
-  const char* kbase = a.pool_k + static_cast<int64_t>(hc) * a.n_slots * ROWB + col * 16;
-  const char* vbase = a.pool_v + static_cast<int64_t>(hc) * a.n_slots * ROWB + col * 16;
+  // cache head of the workgroup's first K row and of its V row; with kPerHeadK the group's K heads
+  // follow at head_stride
+  const int64_t head_stride = a.n_slots * ROWB;
+  const char* kbase = a.pool_k + static_cast<int64_t>(kPerHeadK ? hc * G : hc) * head_stride + col * 16;
+  const char* vbase = a.pool_v + static_cast<int64_t>(kPerHeadK ? hc * G : hc) * head_stride + col * 16;
 
   // page ids of the split -> LDS, then the rows.  Outside row mode one round covers the split.
   int64_t blk0;
@@ -357,7 +370,7 @@ __global__ __launch_bounds__(kThreads) void paged_decode_kernel(const DecodeArgs
 
 #pragma nounroll
   for (int c0 = s0 + wave * CH; c0 < c_end; c0 += kWaves * CH) {
-    v4u kreg[U], vreg[U];
+    v4u kreg[GK][U], vreg[U];
     if (kAligned) {
       // the CH rows of this iteration lie in one page: one base, constant offsets
       const int page = s_pages[(c0 >> a.pd.shift) - static_cast<int>(blk0)];
@@ -366,7 +379,8 @@ __global__ __launch_bounds__(kThreads) void paged_decode_kernel(const DecodeArgs
       const char* vp = vbase + slot * ROWB;
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        kreg[u] = stream_load(kp + u * RPW * ROWB);
+#pragma unroll
+        for (int gk = 0; gk < GK; ++gk) kreg[gk][u] = stream_load(kp + gk * head_stride + u * RPW * ROWB);
         vreg[u] = stream_load(vp + u * RPW * ROWB);
       }
     } else {
@@ -378,14 +392,15 @@ __global__ __launch_bounds__(kThreads) void paged_decode_kernel(const DecodeArgs
         int off;
         a.pd.split(t, blk, off);
         const int64_t slot = static_cast<int64_t>(s_pages[blk - blk0]) * a.pd.page_size + off;
-        kreg[u] = stream_load(kbase + slot * ROWB);
+#pragma unroll
+        for (int gk = 0; gk < GK; ++gk) kreg[gk][u] = stream_load(kbase + gk * head_stride + slot * ROWB);
         vreg[u] = stream_load(vbase + slot * ROWB);
       }
     }
     if (c0 + CH <= c_end)
-      fold_rows<E, TPR, G, U, RPW, false>(kreg, vreg, q, a.qscale, c0 + grp, c_end, m, l, acc);
+      fold_rows<E, TPR, G, GK, U, RPW, false>(kreg, vreg, q, a.qscale, c0 + grp, c_end, m, l, acc);
     else
-      fold_rows<E, TPR, G, U, RPW, true>(kreg, vreg, q, a.qscale, c0 + grp, c_end, m, l, acc);
+      fold_rows<E, TPR, G, GK, U, RPW, true>(kreg, vreg, q, a.qscale, c0 + grp, c_end, m, l, acc);
   }
     if (!kRowMode || s1 >= t1) break;
     __syncthreads();  // every wavefront is done with the page list before it is refilled
@@ -394,22 +409,33 @@ __global__ __launch_bounds__(kThreads) void paged_decode_kernel(const DecodeArgs
 
   if (t1_pool != t1 && wave == 0) {
     // the newest token: one row, held by lane group 0; every other row of this pass is masked
-    v4u kreg[U], vreg[U];
-    const v4u kn = *reinterpret_cast<const v4u*>(a.k_new + b * a.kn_b + hc * a.kn_h + col * 16);
-    const v4u vn = *reinterpret_cast<const v4u*>(a.v_new + b * a.vn_b + hc * a.vn_h + col * 16);
+    v4u kreg[GK][U], vreg[U];
+    const int h0 = kPerHeadK ? hc * G : hc;  // first cache head of this workgroup
+    v4u kn[GK];
+#pragma unroll
+    for (int gk = 0; gk < GK; ++gk)
+      kn[gk] = *reinterpret_cast<const v4u*>(a.k_new + b * a.kn_b + (h0 + gk) * a.kn_h + col * 16);
+    const v4u vn = *reinterpret_cast<const v4u*>(a.v_new + b * a.vn_b + h0 * a.vn_h + col * 16);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      kreg[u] = kn;
+#pragma unroll
+      for (int gk = 0; gk < GK; ++gk) kreg[gk][u] = kn[gk];
       vreg[u] = vn;
     }
-    fold_rows<E, TPR, G, U, RPW, true>(kreg, vreg, q, a.qscale, t1 - 1 + grp, t1, m, l, acc);
+    fold_rows<E, TPR, G, GK, U, RPW, true>(kreg, vreg, q, a.qscale, t1 - 1 + grp, t1, m, l, acc);
     if (grp == 0) {
       int64_t blk;
       int off;
       a.pd.split(t1 - 1, blk, off);
       const int64_t slot = static_cast<int64_t>(s_pages[blk - blk0]) * a.pd.page_size + off;
-      __builtin_nontemporal_store(kn, reinterpret_cast<v4u*>(const_cast<char*>(kbase) + slot * ROWB));
-      __builtin_nontemporal_store(vn, reinterpret_cast<v4u*>(const_cast<char*>(vbase) + slot * ROWB));
+#pragma unroll
+      for (int gk = 0; gk < GK; ++gk) {
+        // every cached head gets its K row; V is written to every copy so the pool stays what the
+        // reference's append leaves (the copies are read by the prefill kernel and by other callers)
+        __builtin_nontemporal_store(kn[gk], reinterpret_cast<v4u*>(const_cast<char*>(kbase) + gk * head_stride + slot * ROWB));
+        const v4u vrow = kPerHeadK ? *reinterpret_cast<const v4u*>(a.v_new + b * a.vn_b + (h0 + gk) * a.vn_h + col * 16) : vn;
+        __builtin_nontemporal_store(vrow, reinterpret_cast<v4u*>(const_cast<char*>(vbase) + gk * head_stride + slot * ROWB));
+      }
     }
   }
 
@@ -505,25 +531,25 @@ __global__ __launch_bounds__(64) void paged_decode_merge_kernel(const DecodeArgs
 constexpr int kPhasePartial = 1;
 constexpr int kPhaseMerge = 2;
 
-template <typename E, int D, int G>
+template <typename E, int D, int G, bool kPerHeadK = false>
 void launch_decode(const DecodeArgs& a, int B, int phases, hipStream_t st) {
-  dim3 grid(a.Hc, B, a.n_splits);
-  // rows per wavefront iteration: 8 loads of 64 / (D * elem / 16) rows each
-  const int chunk_rows = 8 * 64 / (D * static_cast<int>(sizeof(typename E::type)) / 16);
+  dim3 grid(a.Hc, B, a.n_splits);  // a.Hc = workgroups per sequence and split: cache heads, or groups of G heads
+  // rows per wavefront iteration: the loads in flight times 64 / (D * elem / 16) rows each
+  const int chunk_rows = decode_loads_in_flight(G, kPerHeadK) * 64 / (D * static_cast<int>(sizeof(typename E::type)) / 16);
   const bool aligned = a.pd.shift >= 0 && a.pd.page_size % chunk_rows == 0;
   if (a.n_splits == 1) {
     // one split covers every context: the partial pass writes out and lse itself
     if (!(phases & kPhasePartial)) return;
     if (aligned)
-      hipLaunchKernelGGL((paged_decode_kernel<E, D, G, true, true>), grid, dim3(kThreads), 0, st, a);
+      hipLaunchKernelGGL((paged_decode_kernel<E, D, G, true, true, false, kPerHeadK>), grid, dim3(kThreads), 0, st, a);
     else
-      hipLaunchKernelGGL((paged_decode_kernel<E, D, G, true, false>), grid, dim3(kThreads), 0, st, a);
+      hipLaunchKernelGGL((paged_decode_kernel<E, D, G, true, false, false, kPerHeadK>), grid, dim3(kThreads), 0, st, a);
   } else {
     if (phases & kPhasePartial) {
       if (aligned)
-        hipLaunchKernelGGL((paged_decode_kernel<E, D, G, false, true>), grid, dim3(kThreads), 0, st, a);
+        hipLaunchKernelGGL((paged_decode_kernel<E, D, G, false, true, false, kPerHeadK>), grid, dim3(kThreads), 0, st, a);
       else
-        hipLaunchKernelGGL((paged_decode_kernel<E, D, G, false, false>), grid, dim3(kThreads), 0, st, a);
+        hipLaunchKernelGGL((paged_decode_kernel<E, D, G, false, false, false, kPerHeadK>), grid, dim3(kThreads), 0, st, a);
     }
     if (phases & kPhaseMerge)
       hipLaunchKernelGGL((paged_decode_merge_kernel<E, D>), dim3(a.Hq, B), dim3(64), 0, st, a);
@@ -531,7 +557,14 @@ void launch_decode(const DecodeArgs& a, int B, int phases, hipStream_t st) {
 }
 
 template <typename E, int D>
-int dispatch_group(const DecodeArgs& a, int B, int phases, hipStream_t st) {
+int dispatch_group(const DecodeArgs& a, int B, int phases, int kv_rep, hipStream_t st) {
+  if (kv_rep > 1) {  // a.Hc already counts groups of kv_rep heads
+    switch (kv_rep) {
+      case 2: launch_decode<E, D, 2, true>(a, B, phases, st); return FP_OK;
+      case 4: launch_decode<E, D, 4, true>(a, B, phases, st); return FP_OK;
+      default: return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_decode: kv_rep = %d (supported: 1, 2, 4)", kv_rep);
+    }
+  }
   switch (a.Hq / a.Hc) {
     case 1: launch_decode<E, D, 1>(a, B, phases, st); return FP_OK;
     case 2: launch_decode<E, D, 2>(a, B, phases, st); return FP_OK;
@@ -542,10 +575,10 @@ int dispatch_group(const DecodeArgs& a, int B, int phases, hipStream_t st) {
 }
 
 template <typename E>
-int dispatch_dim(const DecodeArgs& a, int B, int D, int phases, hipStream_t st) {
+int dispatch_dim(const DecodeArgs& a, int B, int D, int phases, int kv_rep, hipStream_t st) {
   switch (D) {
-    case 64: return dispatch_group<E, 64>(a, B, phases, st);
-    case 128: return dispatch_group<E, 128>(a, B, phases, st);
+    case 64: return dispatch_group<E, 64>(a, B, phases, kv_rep, st);
+    case 128: return dispatch_group<E, 128>(a, B, phases, kv_rep, st);
     default: return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_decode: head_dim %d (supported: 64, 128)", D);
   }
 }
@@ -616,7 +649,7 @@ int decode_entry(int phases, const NewRows* fresh, const void* q, int64_t q_stri
                  const void* pool_v, const int64_t* page_table, int64_t pt_row_stride,
                  const int64_t* batch_idx, const void* input_pos, int pos_index_type,
                  void* out, int64_t out_stride_b, int64_t out_stride_h, float* lse, const float* sinks,
-                 void* workspace, int64_t workspace_bytes, int32_t B, int32_t Hq, int32_t Hc,
+                 void* workspace, int64_t workspace_bytes, int32_t B, int32_t Hq, int32_t Hc, int32_t kv_rep,
                  int32_t D, int32_t page_size, int32_t n_pages, int32_t max_batch,
                  int64_t n_slots, int32_t max_context, int32_t split_tokens, float scale,
                  int dtype, void* stream) {
@@ -626,6 +659,12 @@ int decode_entry(int phases, const NewRows* fresh, const void* q, int64_t q_stri
       n_slots <= 0 || max_context < 0 || split_tokens < 0)
     return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: bad dimension");
   if (Hq % Hc) return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: Hq=%d not a multiple of Hc=%d", Hq, Hc);
+  if (kv_rep < 1) return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: kv_rep must be at least 1");
+  if (kv_rep > 1 && (Hc != Hq || Hq % kv_rep))
+    return fp::fail(FP_ERR_INVALID_ARGUMENT,
+                    "fp_paged_decode: kv_rep = %d needs a cache with one head per query head (Hc = Hq = %d here %d) "
+                    "and Hq a multiple of kv_rep", kv_rep, Hq, Hc);
+  const int wg_heads = kv_rep > 1 ? Hq / kv_rep : Hc;  // workgroups per sequence and split
   if (n_slots < page_size)
     return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: n_slots smaller than one page");
   if (max_context > static_cast<int64_t>(n_pages) * page_size)
@@ -642,7 +681,7 @@ int decode_entry(int phases, const NewRows* fresh, const void* q, int64_t q_stri
     return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: q and pool rows must be 16-byte aligned");
   if (!fp::aligned(out, eb)) return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: out misaligned");
 
-  if (split_tokens == 0) split_tokens = default_split_tokens(B, Hc, max_context, page_size);
+  if (split_tokens == 0) split_tokens = default_split_tokens(B, wg_heads, max_context, page_size);
   if (split_tokens % 64) return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: split_tokens must be a multiple of 64");
   if (split_tokens / page_size + 2 > kMaxSplitPages)
     return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_decode: split of %d tokens spans more than %d pages", split_tokens,
@@ -654,7 +693,7 @@ int decode_entry(int phases, const NewRows* fresh, const void* q, int64_t q_stri
                static_cast<const char*>(pool_k), static_cast<const char*>(pool_v),
                page_table, pt_row_stride, batch_idx, input_pos, pos_index_type == FP_INDEX_I64,
                static_cast<char*>(out), out_stride_b * eb, out_stride_h * eb, lse, 0, sinks,
-               nullptr, nullptr, Hq, Hc, fp::PageDiv(page_size), n_pages, max_batch, n_slots,
+               nullptr, nullptr, Hq, wg_heads, fp::PageDiv(page_size), n_pages, max_batch, n_slots,
                max_context, split_tokens, ns, scale * kLog2e,  // scores are kept in log2 units
                nullptr, nullptr, 0, 0, 0, 0};
   if (fresh) {
@@ -681,9 +720,9 @@ int decode_entry(int phases, const NewRows* fresh, const void* q, int64_t q_stri
   hipStream_t st = static_cast<hipStream_t>(stream);
   int rc;
   switch (dtype) {
-    case FP_DTYPE_F32: rc = dispatch_dim<F32>(a, B, D, phases, st); break;
-    case FP_DTYPE_BF16: rc = dispatch_dim<BF16>(a, B, D, phases, st); break;
-    default: rc = dispatch_dim<F16>(a, B, D, phases, st); break;
+    case FP_DTYPE_F32: rc = dispatch_dim<F32>(a, B, D, phases, kv_rep, st); break;
+    case FP_DTYPE_BF16: rc = dispatch_dim<BF16>(a, B, D, phases, kv_rep, st); break;
+    default: rc = dispatch_dim<F16>(a, B, D, phases, kv_rep, st); break;
   }
   if (rc != FP_OK) return rc;
   return fp::check_launch("fp_paged_decode");
@@ -696,12 +735,13 @@ int decode_entry(int phases, const NewRows* fresh, const void* q, int64_t q_stri
       const int64_t *page_table, int64_t pt_row_stride, const int64_t *batch_idx, const void *input_pos,  \
       int pos_index_type, void *out, int64_t out_stride_b, int64_t out_stride_h, float *lse,              \
       const float *sinks,                                                                                 \
-      void *workspace, int64_t workspace_bytes, int32_t B, int32_t Hq, int32_t Hc, int32_t D,             \
+      void *workspace, int64_t workspace_bytes, int32_t B, int32_t Hq, int32_t Hc, int32_t kv_rep,        \
+      int32_t D,                                                                                          \
       int32_t page_size, int32_t n_pages, int32_t max_batch, int64_t n_slots, int32_t max_context,        \
       int32_t split_tokens, float scale, int dtype, void *stream
 #define FP_DECODE_ARGS                                                                                     \
   q, q_stride_b, q_stride_h, pool_k, pool_v, page_table, pt_row_stride, batch_idx, input_pos,             \
-      pos_index_type, out, out_stride_b, out_stride_h, lse, sinks, workspace, workspace_bytes, B, Hq, Hc, D, \
+      pos_index_type, out, out_stride_b, out_stride_h, lse, sinks, workspace, workspace_bytes, B, Hq, Hc, kv_rep, D, \
       page_size, n_pages, max_batch, n_slots, max_context, split_tokens, scale, dtype, stream
 
 extern "C" int fp_paged_decode(FP_DECODE_PARAMS) {

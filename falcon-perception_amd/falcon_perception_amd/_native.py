@@ -44,7 +44,7 @@ SIGNATURES = {
         c_void_p, c_int64, c_void_p, c_void_p, c_int,
         c_void_p, c_int64, c_int64, c_void_p, c_void_p,
         c_void_p, c_int64,
-        c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
+        c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
         c_int64, c_int32, c_int32, c_float, c_int, c_void_p]),
     "fp_paged_decode_partial": None,  # same signature as fp_paged_decode, filled in below
     "fp_paged_decode_merge": None,

@@ -182,12 +182,14 @@ def compiled_flex_attn_decode(q: Tensor, k: Tensor, v: Tensor, score_mod=None, b
         raise RuntimeError("paged decode attention called before PagedKVCache.insert_kv for this step")
     if q.shape[2] != 1:
         raise RuntimeError("a PagedDecodeMask serves one query token per sequence")
+    kv_rep = getattr(cache, "kv_rep", 1)
+    wg_heads = k.shape[1] // kv_rep  # workgroups per sequence and split
     out, lse = ops.paged_decode(
         q, k[0], v[0], cache.page_table, block_mask.batch_idx, step.input_pos,
         cache.page_size, block_mask.max_context, scale=scale,
-        workspace=cache.decode_workspace(q.shape[0], q.shape[1], q.shape[3], block_mask.max_context, k.shape[1]),
-        split_tokens=cache.decode_split_tokens(q.shape[0], k.shape[1], block_mask.max_context),
-        sinks=sinks,
+        workspace=cache.decode_workspace(q.shape[0], q.shape[1], q.shape[3], block_mask.max_context, wg_heads),
+        split_tokens=cache.decode_split_tokens(q.shape[0], wg_heads, block_mask.max_context),
+        sinks=sinks, kv_rep=kv_rep,
     )
     return _result(out, lse, return_aux, return_lse)
 

@@ -175,8 +175,11 @@ def paged_decode(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor, 
                  split_tokens: int = 0, workspace: Tensor | None = None,
                  out: Tensor | None = None, lse: Tensor | None = None, phase: str = "both",
                  k_new: Tensor | None = None, v_new: Tensor | None = None,
-                 sinks: Tensor | None = None) -> tuple[Tensor, Tensor]:
+                 sinks: Tensor | None = None, kv_rep: int = 1) -> tuple[Tensor, Tensor]:
     """Single-query paged attention.  q [B, Hq, 1, D]; pools [Hc, N, D]; returns out [B, Hq, 1, D], lse [B, Hq, 1].
+
+    `kv_rep` > 1 declares a cache with one head per query head whose V heads are `kv_rep` identical
+    copies (the reference's `repeat_kv` layout, `model.py:112-114`): V is then read once per group.
 
     With `sinks` [Hq] float32 the output is gated as the reference's `_post_attention` does
     (model.py:122-128): out * sigmoid(lse - sinks[h]); lse is returned ungated.
@@ -199,7 +202,7 @@ def paged_decode(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor, 
     if scale is None:
         scale = 1.0 / math.sqrt(D)
     if split_tokens == 0:
-        split_tokens = decode_split_tokens(B, Hc, max_context, page_size)
+        split_tokens = decode_split_tokens(B, Hc // kv_rep if kv_rep > 1 else Hc, max_context, page_size)
     need = decode_workspace_bytes(B, Hq, D, max_context, split_tokens)
     if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
         workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
@@ -229,7 +232,7 @@ def paged_decode(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor, 
         out.data_ptr(), out.stride(0), out.stride(1), lse.data_ptr(), sinks_ptr,
         workspace.data_ptr() if workspace is not None else None,
         workspace.numel() * workspace.element_size() if workspace is not None else 0,
-        B, Hq, Hc, D, page_size, page_table.shape[1], page_table.shape[0],
+        B, Hq, Hc, kv_rep, D, page_size, page_table.shape[1], page_table.shape[0],
         n_slots, max_context, split_tokens, scale, N.dtype_code(q.dtype), N.stream_ptr(q.device))
     N.check(rc, entry)
     return out, lse

@@ -77,6 +77,10 @@ class PagedKVCache(KVCacheBase):
         self.kv_shape = (num_layers, 2, 1, n_heads, n_pages * page_size, head_dim)
         self.kv_cache = torch.zeros(self.kv_shape, dtype=dtype, device=device)
 
+        # 1, or n_heads // n_kv_heads when the cached V heads are plain copies inside a group (the model's
+        # repeat_kv, model.py:112-113): the decode kernel then reads V once per group.  Off unless set.
+        self.kv_rep = 1
+
         # what the attention callables need from the step in flight
         self.last_decode_step: StepMeta | None = None
         self.last_prefill_step: StepMeta | None = None

@@ -153,6 +153,11 @@ int64_t fp_paged_decode_workspace_bytes(int32_t B, int32_t Hq, int32_t D,
  *   input_pos[B] int32/int64: sequence b attends logical positions 0..input_pos[b]
  *   out      [B, Hq, 1, D] same dtype as q, element strides (b, h)
  *   lse      [B, Hq] float32, natural log of the softmax denominator
+ *   kv_rep   1, or (2, 4) for a cache that stores one head per query head (Hc = Hq) whose V heads
+ *            are kv_rep identical copies while the K heads differ -- what the reference's
+ *            repeat_kv before the per-head rotary embedding produces (model.py:112-114).  The
+ *            kernel then reads the kv_rep K rows of a group and one V row (the first copy)
+ *            instead of kv_rep of each; results equal those of kv_rep = 1 on such a cache
  *   sinks    NULL, or [Hq] float32: out is multiplied by sigmoid(lse - sinks[h]), the
  *            attention-sink gate of Attention._post_attention (model.py:122-128), with the
  *            reference's rounding (attention output rounded to the dtype, product rounded again);
@@ -171,7 +176,7 @@ int fp_paged_decode(const void* q, int64_t q_stride_b, int64_t q_stride_h,
                     void* out, int64_t out_stride_b, int64_t out_stride_h,
                     float* lse, const float* sinks,
                     void* workspace, int64_t workspace_bytes,
-                    int32_t B, int32_t Hq, int32_t Hc, int32_t D,
+                    int32_t B, int32_t Hq, int32_t Hc, int32_t kv_rep, int32_t D,
                     int32_t page_size, int32_t n_pages, int32_t max_batch,
                     int64_t n_slots, int32_t max_context, int32_t split_tokens,
                     float scale, int dtype,
@@ -196,7 +201,7 @@ int fp_paged_decode_partial(const void* q, int64_t q_stride_b, int64_t q_stride_
                             void* out, int64_t out_stride_b, int64_t out_stride_h,
                             float* lse, const float* sinks,
                             void* workspace, int64_t workspace_bytes,
-                            int32_t B, int32_t Hq, int32_t Hc, int32_t D,
+                            int32_t B, int32_t Hq, int32_t Hc, int32_t kv_rep, int32_t D,
                             int32_t page_size, int32_t n_pages, int32_t max_batch,
                             int64_t n_slots, int32_t max_context, int32_t split_tokens,
                             float scale, int dtype,
@@ -209,7 +214,7 @@ int fp_paged_decode_merge(const void* q, int64_t q_stride_b, int64_t q_stride_h,
                           void* out, int64_t out_stride_b, int64_t out_stride_h,
                           float* lse, const float* sinks,
                           void* workspace, int64_t workspace_bytes,
-                          int32_t B, int32_t Hq, int32_t Hc, int32_t D,
+                          int32_t B, int32_t Hq, int32_t Hc, int32_t kv_rep, int32_t D,
                           int32_t page_size, int32_t n_pages, int32_t max_batch,
                           int64_t n_slots, int32_t max_context, int32_t split_tokens,
                           float scale, int dtype,
@@ -237,7 +242,7 @@ int fp_paged_decode_append(const void* k_new, const void* v_new,
                            void* out, int64_t out_stride_b, int64_t out_stride_h,
                            float* lse, const float* sinks,
                            void* workspace, int64_t workspace_bytes,
-                           int32_t B, int32_t Hq, int32_t Hc, int32_t D,
+                           int32_t B, int32_t Hq, int32_t Hc, int32_t kv_rep, int32_t D,
                            int32_t page_size, int32_t n_pages, int32_t max_batch,
                            int64_t n_slots, int32_t max_context, int32_t split_tokens,
                            float scale, int dtype,
