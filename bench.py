@@ -349,6 +349,34 @@ def graph_ms(fn, steps: int) -> float:
     return (time.perf_counter() - t0) * 1e3 / steps
 
 
+def model_depth_graph_ms(case: "DecodeCase", steps: int, layers: int = MODEL_LAYERS) -> float | None:
+    """ms for the fused decode step of ALL layers of the model, replayed from one captured HIP graph: every
+    layer has its own K/V planes (the same page table, as in the engine) so nothing is served from cache
+    between layers.  None when the planes do not fit next to the case's own pool."""
+    from falcon_perception_amd import ops
+
+    c = case.cfg
+    plane = case.pool_k.numel() * case.pool_k.element_size()
+    free, _ = torch.cuda.mem_get_info()
+    if 2 * plane * layers > free - (8 << 30):
+        return None
+    pools = torch.empty((layers, 2) + tuple(case.pool_k.shape), dtype=case.pool_k.dtype, device=case.pool_k.device)
+    for layer in range(layers):
+        pools[layer, 0].copy_(case.pool_k)
+        pools[layer, 1].copy_(case.pool_v)
+
+    def all_layers():
+        for layer in range(layers):
+            ops.paged_decode(case.q, pools[layer, 0], pools[layer, 1], case.cache.page_table, case.batch_idx,
+                             case.input_pos, case.page_size, case.max_context, split_tokens=case.split_tokens,
+                             workspace=case.workspace, out=case.out, lse=case.lse, k_new=case.k_new, v_new=case.v_new,
+                             kv_rep=c.get("kv_rep", 1))
+
+    ms = graph_ms(all_layers, max(steps // 10, 5))
+    del pools
+    return ms
+
+
 def append_gather_rates(steps: int = 20, T: int = 32768, H: int = 16, D: int = 128, P: int = 128) -> dict:
     """KV append and page gather at a prefill-sized batch of tokens (the engine's prefill limit,
     reference paged_inference.py:233): bf16, 16 stored heads, one fragmented page table."""
@@ -526,6 +554,7 @@ def main() -> int:
     ms_separate = time_steps(case.run, args.steps, args.warmup)
     ms_gated = time_steps(case.run_fused_gated, args.steps, args.warmup)
     ms_graph = graph_ms(case.run_fused, args.steps)
+    ms_model = None if args.decode_only else model_depth_graph_ms(case, args.steps)
     ms_decode = event_ms(case.attend, args.steps)
     ms_partial = event_ms(lambda: case.attend("partial"), args.steps)  # the dominant kernel alone
     ms_merge = event_ms(lambda: case.attend("merge"), args.steps)
@@ -550,6 +579,9 @@ def main() -> int:
         "pct_of_hbm_peak": 100.0 * value / HBM_PEAK_GBPS,
         "decode_tok_s_per_layer": c["B"] / (ms_step * 1e-3),
         "decode_tok_s_model": c["B"] / (ms_step * 1e-3) / MODEL_LAYERS,
+        # measured, not divided: the fused step of all 28 layers (own K/V planes each) in one HIP graph
+        "ms_all_layers_hip_graph": ms_model,
+        "decode_tok_s_model_measured": None if ms_model is None else c["B"] / (ms_model * 1e-3),
         "step": "fp_paged_decode_append (append fused into the split-K pass) + merge pass",
         "ms_per_step_separate_append": ms_separate,
         "ms_per_step_with_sink_gate": ms_gated,  # same step, sigmoid(lse - sink) gate + [B,1,H*D] layout in the merge
