@@ -307,6 +307,7 @@ def make_prefill_case(name: str, device="cuda") -> PrefillCase:
 
 def time_steps(fn, steps: int, warmup: int) -> float:
     """Wall-clock ms per step of `fn`, launches back to back, synchronised on both sides."""
+    warm_clocks(fn)
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -317,8 +318,20 @@ def time_steps(fn, steps: int, warmup: int) -> float:
     return (time.perf_counter() - t0) * 1e3 / steps
 
 
+def warm_clocks(fn, seconds: float = 0.2) -> None:
+    """Run `fn` back to back for a while: after an idle spell the shader clock needs some tens of
+    milliseconds of load to come up, and a handful of warm-up calls would be timed on the ramp
+    (a 560 us kernel measured 620 us that way)."""
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
+
+
 def event_ms(fn, steps: int) -> float:
     """Average device ms per call of `fn`, HIP events on the stream the kernels run on."""
+    warm_clocks(fn)
     stream = torch.cuda.current_stream()
     starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
     ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
@@ -342,6 +355,7 @@ def graph_ms(fn, steps: int) -> float:
         fn()
     g.replay()
     torch.cuda.synchronize()
+    warm_clocks(g.replay)
     t0 = time.perf_counter()
     for _ in range(steps):
         g.replay()
@@ -374,6 +388,7 @@ def model_depth_graph_ms(case: "DecodeCase", steps: int, layers: int = MODEL_LAY
 
     ms = graph_ms(all_layers, max(steps // 10, 5))
     del pools
+    torch.cuda.empty_cache()  # hand the 56 GiB back: later allocations carved out of it measured 15 % slower copies
     return ms
 
 
@@ -554,7 +569,6 @@ def main() -> int:
     ms_separate = time_steps(case.run, args.steps, args.warmup)
     ms_gated = time_steps(case.run_fused_gated, args.steps, args.warmup)
     ms_graph = graph_ms(case.run_fused, args.steps)
-    ms_model = None if args.decode_only else model_depth_graph_ms(case, args.steps)
     ms_decode = event_ms(case.attend, args.steps)
     ms_partial = event_ms(lambda: case.attend("partial"), args.steps)  # the dominant kernel alone
     ms_merge = event_ms(lambda: case.attend("merge"), args.steps)
@@ -580,8 +594,8 @@ def main() -> int:
         "decode_tok_s_per_layer": c["B"] / (ms_step * 1e-3),
         "decode_tok_s_model": c["B"] / (ms_step * 1e-3) / MODEL_LAYERS,
         # measured, not divided: the fused step of all 28 layers (own K/V planes each) in one HIP graph
-        "ms_all_layers_hip_graph": ms_model,
-        "decode_tok_s_model_measured": None if ms_model is None else c["B"] / (ms_model * 1e-3),
+        "ms_all_layers_hip_graph": None,
+        "decode_tok_s_model_measured": None,
         "step": "fp_paged_decode_append (append fused into the split-K pass) + merge pass",
         "ms_per_step_separate_append": ms_separate,
         "ms_per_step_with_sink_gate": ms_gated,  # same step, sigmoid(lse - sink) gate + [B,1,H*D] layout in the merge
@@ -599,6 +613,10 @@ def main() -> int:
     if not args.decode_only:
         result["prefill_sized"] = append_gather_rates()
         result["chunked_prefill"] = prefill_rate()
+        ms_model = model_depth_graph_ms(case, args.steps)  # last: it takes and returns 56 GiB
+        if ms_model is not None:
+            result["ms_all_layers_hip_graph"] = ms_model
+            result["decode_tok_s_model_measured"] = c["B"] / (ms_model * 1e-3)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(case)
         result["gpu_over_cpu"] = value / result["cpu_baseline"]["value"]
