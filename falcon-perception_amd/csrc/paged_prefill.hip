@@ -33,7 +33,8 @@ constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * 64;
 constexpr int kTileN = 64;  // keys per tile
 constexpr float kMaxSlack = 6.f;  // the running maximum may lag a row's true maximum by this much (log2)
-constexpr int kPrefetch = 3; // LDS operand reads in flight ahead of the MFMA that uses them
+constexpr int kPrefetchK = 6; // K operand reads in flight ahead of the MFMA that uses them
+constexpr int kPrefetchV = 4; // V^T operand read pairs in flight ahead of their MFMA
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
@@ -110,6 +111,17 @@ template <int N>
 struct IntC {
   static constexpr int value = N;
 };
+
+// 16 bytes per lane from global memory straight into LDS at `lds` + lane * 16 (`lds` wavefront-uniform).
+// Written as inline assembly on purpose: while the compiler knows of such a load in flight it turns
+// every wait for an LDS read into a wait for all of them, which serialises the operand reads of the
+// main loop against the MFMAs.  The code that issues these loads waits for them itself (vmcnt(0)
+// before the barrier that publishes a tile).
+__device__ __forceinline__ void load_to_lds(const char* src, char* lds) {
+  const uint32_t base = __builtin_amdgcn_readfirstlane(
+      static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds)));
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(base), "v"(src) : "memory", "m0");
+}
 
 // K/V tiles in LDS are 64 unpadded rows of D * 2 bytes, filled by global_load_lds (each lane's
 // 16 bytes land at base + lane * 16).  Bank conflicts are avoided by permuting the 16-byte chunks
@@ -322,11 +334,9 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
       const int i = piece >> 1;
       const int group = (i * kWaves + wave) * RPI * ROWB;  // wavefront-uniform LDS offset
       if ((piece & 1) == 0)
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(ksrc + rowbyte[i]),
-                                         (__attribute__((address_space(3))) void*)(kdst + group), 16, 0, 0);
+        load_to_lds(ksrc + rowbyte[i], kdst + group);
       else
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(vsrc + rowbyte[i]),
-                                         (__attribute__((address_space(3))) void*)(vdst + group), 16, 0, 0);
+        load_to_lds(vsrc + rowbyte[i], vdst + group);
     };
     auto fetch = [&](char* kdst, char* vdst) {
 #pragma unroll
@@ -366,22 +376,26 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
       if (work) {
         f32x16 s_acc[MB][2];  // written by the first MFMA of each block, which starts from zero
         // ---- S^T = K Q^T for the two 32-key blocks of the tile ----
-        // LDS operands are read kPrefetch steps ahead of the MFMA that consumes them
+        // LDS operands are read kPrefetchK steps ahead of the MFMA that consumes them; the two 32-key
+        // blocks alternate so that consecutive MFMAs are independent.  The scheduling barriers pin this
+        // order: left alone, the compiler gathers the reads and waits for all of them before every MFMA.
         auto read_k = [&](int t) {
-          const int kb = t / DS, ds = t % DS;
+          const int kb = t & 1, ds = t >> 1;
           return *reinterpret_cast<const v4u*>(kcur + kofs[ds] + kb * 32 * ROWB);
         };
-        v4u ring[kPrefetch];
+        v4u ring[kPrefetchK];
 #pragma unroll
-        for (int t = 0; t < kPrefetch; ++t) ring[t] = read_k(t);
+        for (int t = 0; t < kPrefetchK; ++t) ring[t] = read_k(t);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int t = 0; t < 2 * DS; ++t) {
-          const s16x8 ka = __builtin_bit_cast(s16x8, ring[t % kPrefetch]);
-          if (t + kPrefetch < 2 * DS) ring[t % kPrefetch] = read_k(t + kPrefetch);
+          const s16x8 ka = __builtin_bit_cast(s16x8, ring[t % kPrefetchK]);
           if (t % kIssueEvery == 0) fetch_piece(t / kIssueEvery, k1, v1);
 #pragma unroll
           for (int mb = 0; mb < MB; ++mb)
-            s_acc[mb][t / DS] = E::mfma(ka, qreg[mb][t % DS], t % DS == 0 ? kZero16 : s_acc[mb][t / DS]);
+            s_acc[mb][t & 1] = E::mfma(ka, qreg[mb][t >> 1], (t >> 1) == 0 ? kZero16 : s_acc[mb][t & 1]);
+          if (t + kPrefetchK < 2 * DS) ring[t % kPrefetchK] = read_k(t + kPrefetchK);
+          __builtin_amdgcn_sched_barrier(0);
         }
 
         // ---- online softmax, one query per lane ----
@@ -452,16 +466,18 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
             lo = lds_read_tr(p0);
             hi = lds_read_tr(p0 + 8 * ROWB);
           };
-          s16x4 rlo[kPrefetch], rhi[kPrefetch];
+          s16x4 rlo[kPrefetchV], rhi[kPrefetchV];
 #pragma unroll
-          for (int t = 0; t < kPrefetch; ++t) read_v(t, rlo[t], rhi[t]);
+          for (int t = 0; t < kPrefetchV; ++t) read_v(t, rlo[t], rhi[t]);
+          __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
           for (int t = 0; t < 4 * DB; ++t) {
-            const s16x4 lo = rlo[t % kPrefetch], hi = rhi[t % kPrefetch];
+            const s16x4 lo = rlo[t % kPrefetchV], hi = rhi[t % kPrefetchV];
             const s16x8 va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-            if (t + kPrefetch < 4 * DB) read_v(t + kPrefetch, rlo[t % kPrefetch], rhi[t % kPrefetch]);
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) o_acc[mb][t % DB] = E::mfma(va, p_op[mb][t / DB], o_acc[mb][t % DB]);
+            if (t + kPrefetchV < 4 * DB) read_v(t + kPrefetchV, rlo[t % kPrefetchV], rhi[t % kPrefetchV]);
+            __builtin_amdgcn_sched_barrier(0);
           }
         }
       }
