@@ -32,8 +32,9 @@ namespace {
 constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * 64;
 constexpr int kTileN = 64;  // keys per tile
+constexpr int kSlotTable = 2048;  // tiles of a run whose first pool slot is looked up ahead of the tile loop
 constexpr float kMaxSlack = 6.f;  // the running maximum may lag a row's true maximum by this much (log2)
-constexpr int kPrefetchK = 6; // K operand reads in flight ahead of the MFMA that uses them
+constexpr int kPrefetchK = 4; // K operand reads in flight ahead of the MFMA that uses them
 constexpr int kPrefetchV = 4; // V^T operand read pairs in flight ahead of their MFMA
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
@@ -120,7 +121,14 @@ struct IntC {
 __device__ __forceinline__ void load_to_lds(const char* src, char* lds) {
   const uint32_t base = __builtin_amdgcn_readfirstlane(
       static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds)));
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(base), "v"(src) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(base), "v"(src) : "memory");
+}
+
+// The same with the address split into a wavefront-uniform base (scalar registers) and a 32-bit offset per lane.
+__device__ __forceinline__ void load_to_lds(const char* base, uint32_t offset, char* lds) {
+  const uint32_t m0v = __builtin_amdgcn_readfirstlane(
+      static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds)));
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(m0v), "v"(offset), "s"(base) : "memory");
 }
 
 // K/V tiles in LDS are 64 unpadded rows of D * 2 bytes, filled by global_load_lds (each lane's
@@ -165,6 +173,7 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
   __shared__ __attribute__((aligned(1024))) char s_v1[TILE_BYTES];
   __shared__ int s_bidx[BM];
   __shared__ int s_red[kWaves];
+  __shared__ int s_tslot[kSlotTable];
 
   // linear id = cache head + Hc * tile: all tiles that read one cache head run on the XCD that
   // already holds its K/V in L2
@@ -287,15 +296,33 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
     }
 
     // ---- K/V fetch pipeline ----
-    // Every wavefront stages NI groups of RPI rows of each tile.  Page ids are loaded a tile
-    // before they are needed and turned into row addresses right after a barrier, where every
-    // load of this wavefront has landed anyway; the staging loads themselves then need no wait.
-    // A key that does not exist (past the run's last key, or an unmapped page) reads slot 0:
-    // finite bytes, and every such key is masked.  Tiles past the last one are staged the same
-    // way (all rows from slot 0) so the loop carries no "is there a next tile" branches.
+    // Every wavefront stages NI groups of RPI rows of each tile.  Where a page holds whole tiles
+    // (page size a power of two, at least the tile), a tile that lies before the run's last key in a
+    // mapped page is contiguous in the pool: its first slot is looked up once per run into s_tslot,
+    // and a staging load is then a scalar base plus a fixed offset per lane.  Any other tile (the
+    // last one of a run, small or odd page sizes, unmapped pages, runs longer than the table) is
+    // staged row by row: a key that does not exist (past the run's last key, or an unmapped page)
+    // reads slot 0, finite bytes, and every such key is masked.
     const int64_t* pt_row = a.page_table + static_cast<int64_t>(sq) * a.pt_row_stride;
-    int64_t page_next[NI];  // page ids of the rows this lane stages next, as loaded
-    int64_t rowbyte[NI];    // byte offset of those rows inside a head's plane
+    const int64_t pool_pages = a.n_slots / a.pd.page_size;
+    const bool page_holds_tile = kPow2 && a.pd.page_size % kTileN == 0;
+    for (int t = tid; t < n_kv_tiles && t < kSlotTable; t += kThreads) {
+      int slot = -1;
+      if (page_holds_tile && (t + 1) * kTileN <= kv_max) {
+        const int key0 = t * kTileN;
+        const int blk = key0 >> a.pd.shift;
+        if (blk < a.n_pages) {
+          const int64_t pg = pt_row[blk];
+          if (pg >= 0 && pg < pool_pages) slot = static_cast<int>(pg) * a.pd.page_size + (key0 & (a.pd.page_size - 1));
+        }
+      }
+      s_tslot[t] = slot;
+    }
+    __syncthreads();
+    // first pool slot of tile kt, or -1: wavefront-uniform
+    auto tile_slot = [&](int kt) {
+      return __builtin_amdgcn_readfirstlane((kt >= 0 && kt < n_kv_tiles && kt < kSlotTable) ? s_tslot[kt] : -1);
+    };
 
     auto key_block = [&](int kpos, int& blkid, int& off) {
       if (kPow2) {  // page size is a power of two: shift and mask, no branch on the page size
@@ -306,41 +333,34 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
         off = kpos - blkid * a.pd.page_size;
       }
     };
-    auto lookup = [&](int kt) {
-#pragma unroll
-      for (int i = 0; i < NI; ++i) {
-        const int kpos = kt * kTileN + i * kWaves * RPI + st_row0;
-        int blkid, off;
-        key_block(kpos, blkid, off);
-        page_next[i] = pt_row[(kpos < kv_max && blkid < a.n_pages) ? blkid : 0];
-      }
-    };
-    const int64_t pool_pages = a.n_slots / a.pd.page_size;
-    auto resolve = [&](int kt) {  // page_next holds the ids of tile kt
-#pragma unroll
-      for (int i = 0; i < NI; ++i) {
-        const int kpos = kt * kTileN + i * kWaves * RPI + st_row0;
-        int blkid, off;
-        key_block(kpos, blkid, off);
-        const bool ok = kpos < kv_max && blkid < a.n_pages && page_next[i] >= 0 && page_next[i] < pool_pages;
-        const int slot = ok ? static_cast<int>(page_next[i]) * a.pd.page_size + off : 0;
-        rowbyte[i] = static_cast<int64_t>(slot) * ROWB;
-      }
-    };
     const char* ksrc = kplane + k_src_off;
     const char* vsrc = vplane + v_src_off;
-    // One staging load: piece 2 * i is the K load of row group i, piece 2 * i + 1 its V load.
-    auto fetch_piece = [&](int piece, char* kdst, char* vdst) {
-      const int i = piece >> 1;
-      const int group = (i * kWaves + wave) * RPI * ROWB;  // wavefront-uniform LDS offset
-      if ((piece & 1) == 0)
-        load_to_lds(ksrc + rowbyte[i], kdst + group);
-      else
-        load_to_lds(vsrc + rowbyte[i], vdst + group);
-    };
-    auto fetch = [&](char* kdst, char* vdst) {
+    uint32_t lane_k[NI], lane_v[NI];  // byte offset of this lane's 16 bytes from the first row of a tile
 #pragma unroll
-      for (int piece = 0; piece < 2 * NI; ++piece) fetch_piece(piece, kdst, vdst);
+    for (int i = 0; i < NI; ++i) {
+      lane_k[i] = (i * kWaves * RPI + st_row0) * ROWB + k_src_off;
+      lane_v[i] = (i * kWaves * RPI + st_row0) * ROWB + v_src_off;
+    }
+    // One staging load of tile kt, whose first slot is ts (or -1): pieces 0 .. NI - 1 are the V loads
+    // of the row groups, NI .. 2 NI - 1 the K loads.  Tiles past the run's last one are not staged.
+    auto fetch_piece = [&](int piece, int kt, int ts, char* dst) {
+      if (kt >= n_kv_tiles) return;
+      const int i = piece % NI;
+      const bool is_k = piece >= NI;
+      char* lds = dst + (i * kWaves + wave) * RPI * ROWB;  // wavefront-uniform
+      if (ts >= 0) {
+        load_to_lds((is_k ? kplane : vplane) + static_cast<int64_t>(ts) * ROWB, is_k ? lane_k[i] : lane_v[i], lds);
+      } else {
+        asm volatile("");  // rare: keep it out of the way as a branch
+        const int kpos = kt * kTileN + i * kWaves * RPI + st_row0;
+        int blkid, off;
+        key_block(kpos, blkid, off);
+        const bool in_range = kpos < kv_max && blkid < a.n_pages;
+        const int64_t pg = pt_row[in_range ? blkid : 0];
+        const bool ok = in_range && pg >= 0 && pg < pool_pages;
+        const int slot = ok ? static_cast<int>(pg) * a.pd.page_size + off : 0;
+        load_to_lds((is_k ? ksrc : vsrc) + static_cast<int64_t>(slot) * ROWB, lds);
+      }
     };
 
     // per-lane LDS offsets of the operand reads, the same for every tile and buffer
@@ -351,34 +371,102 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
     for (int db = 0; db < DB; ++db)
       vofs[db] = (half * 4 + (bi >> 2)) * ROWB + (bi & 3) * 8 + ((2 * db + vsel) % R32) * 32;
 
-    lookup(0);
-    resolve(0);
-    fetch(s_k0, s_v0);
-    lookup(1);
+    // ---- schedule ----
+    // Step i of a wavefront is M(i) = { O^T += V^T P^T of tile i - 1;  S^T = K Q^T of tile i } on the
+    // matrix pipe, then X(i) = softmax of tile i on the vector pipe.  The two wavefronts that share a
+    // SIMD (w and w + 4) run half a step apart, held there by two barriers per step: while one is in
+    // M the other is in X, so the matrix and the vector pipe of the SIMD work at the same time.
+    //   barrier 2i     first half: M(i)     second half: X(i - 1)
+    //   barrier 2i+1   first half: X(i)     second half: M(i)
+    // Staging step i (K of tile i + 1, V of tile i) is issued after barrier 2i, when M(i - 1) is over
+    // everywhere, and has landed before barrier 2i + 2, after which M(i + 1) begins.  K(i) lives in
+    // K buffer i % 2, V(i) in V buffer i % 2.
+    {
+      const int ts0 = tile_slot(0);
+#pragma unroll
+      for (int piece = NI; piece < 2 * NI; ++piece) fetch_piece(piece, 0, ts0, s_k0);  // K(0)
+    }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's rows have landed in LDS
-    __syncthreads();
 
-    // one tile: stage tile kt + 1 into the other buffer while working on tile kt
-    auto tile_step = [&](auto parity, int kt) {
+    s16x8 p_op[MB][4];  // P^T as B operands of the 4 k-steps (16 keys each), from X(i) to M(i + 1)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) p_op[mb][j] = s16x8{0, 0, 0, 0, 0, 0, 0, 0};
+
+    float alpha_next[MB];  // factor the accumulators still have to take before tile i - 1 is added
+    bool moved_next[MB];   // whether it differs from 1 (uniform over the wavefront)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      alpha_next[mb] = 1.f;
+      moved_next[mb] = false;
+    }
+    auto step = [&](auto second_c, auto parity, int i) {
+      constexpr bool kSecond = decltype(second_c)::value != 0;
       constexpr int kBuf = decltype(parity)::value;
-      const char* kcur = kBuf ? s_k1 : s_k0;
-      const char* vcur = kBuf ? s_v1 : s_v0;
-      char* k1 = kBuf ? s_k0 : s_k1;
-      char* v1 = kBuf ? s_v0 : s_v1;
-      constexpr int kIssueEvery = DS / NI;  // MFMA steps between two staging loads: 2 * DS steps, 2 * NI pieces
+      const char* kcur = kBuf ? s_k1 : s_k0;   // K(i)
+      const char* vprev = kBuf ? s_v0 : s_v1;  // V(i - 1)
+      char* knext = kBuf ? s_k0 : s_k1;        // K(i + 1) goes here
+      char* vcur = kBuf ? s_v1 : s_v0;         // V(i) goes here
+      const int key0 = i * kTileN;
+      const bool work_cur = key0 < wave_max;
+      const bool work_prev = i > 0 && key0 - kTileN < wave_max;
 
-      const int key0 = kt * kTileN;
-      const bool work = key0 < wave_max;
-      resolve(kt + 1);
-      lookup(kt + 2);
-      if (!work) fetch(k1, v1);  // no arithmetic to hide the loads behind
+      // the staging step this wavefront issues during the step: K of tile kt_k, V of tile kt_k - 1.
+      // The table is read ahead of the barrier, whose wait hides the LDS latency.
+      const int kt_k = kSecond ? i + 2 : i + 1;
+      const int ts_k = tile_slot(kt_k);
+      const int ts_v = tile_slot(kt_k - 1);
+      if (!kSecond) __builtin_amdgcn_s_waitcnt(0x0F70);  // staging step i - 1 of this wavefront has landed
+      __builtin_amdgcn_s_barrier();
 
-      if (work) {
-        f32x16 s_acc[MB][2];  // written by the first MFMA of each block, which starts from zero
-        // ---- S^T = K Q^T for the two 32-key blocks of the tile ----
-        // LDS operands are read kPrefetchK steps ahead of the MFMA that consumes them; the two 32-key
-        // blocks alternate so that consecutive MFMAs are independent.  The scheduling barriers pin this
-        // order: left alone, the compiler gathers the reads and waits for all of them before every MFMA.
+      // ---- M(i), first part: O^T += V^T P^T of tile i - 1 ----
+      f32x16 s_acc[MB][2];  // written by the first MFMA of each block, which starts from zero
+      constexpr int kPvEvery = 4 * DB / NI;  // MFMA steps between two staging loads
+      constexpr int kSEvery = 2 * DS / NI;
+      if (work_prev) {
+        asm volatile("");
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+          if (moved_next[mb]) {
+            asm volatile("");  // the rescale is rare and must not run unconditionally
+#pragma unroll
+            for (int db = 0; db < DB; ++db) o_acc[mb][db] *= alpha_next[mb];
+          }
+        }
+        // step t = (j, db): this lane names the chunk (key = base + bi / 4, d = dblock + 4 * (bi % 4))
+        // and receives d = dblock + bi for keys base .. base + 3, once for each half of the 16 keys
+        auto read_v = [&](int t, s16x4& lo, s16x4& hi) {
+          const int j = t / DB, db = t % DB;
+          const char* p0 = vprev + vofs[db] + ((j >> 1) * 32 + (j & 1) * 16) * ROWB;
+          lo = lds_read_tr(p0);
+          hi = lds_read_tr(p0 + 8 * ROWB);
+        };
+        s16x4 rlo[kPrefetchV], rhi[kPrefetchV];
+#pragma unroll
+        for (int t = 0; t < kPrefetchV; ++t) read_v(t, rlo[t], rhi[t]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < 4 * DB; ++t) {
+          const s16x4 lo = rlo[t % kPrefetchV], hi = rhi[t % kPrefetchV];
+          const s16x8 va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          if (!kSecond && t % kPvEvery == 0) fetch_piece(t / kPvEvery, kt_k - 1, ts_v, vcur);
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb) o_acc[mb][t % DB] = E::mfma(va, p_op[mb][t / DB], o_acc[mb][t % DB]);
+          if (t + kPrefetchV < 4 * DB) read_v(t + kPrefetchV, rlo[t % kPrefetchV], rhi[t % kPrefetchV]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else if (!kSecond) {
+#pragma unroll
+        for (int piece = 0; piece < NI; ++piece) fetch_piece(piece, kt_k - 1, ts_v, vcur);
+      }
+
+      // ---- M(i), second part: S^T = K Q^T for the two 32-key blocks of tile i ----
+      // LDS operands are read kPrefetchK steps ahead of the MFMA that consumes them; the two 32-key
+      // blocks alternate so that consecutive MFMAs are independent.  The scheduling barriers pin this
+      // order: left alone, the compiler gathers the reads and waits for all of them before every MFMA.
+      if (work_cur) {
+        asm volatile("");
         auto read_k = [&](int t) {
           const int kb = t & 1, ds = t >> 1;
           return *reinterpret_cast<const v4u*>(kcur + kofs[ds] + kb * 32 * ROWB);
@@ -390,29 +478,44 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
 #pragma unroll
         for (int t = 0; t < 2 * DS; ++t) {
           const s16x8 ka = __builtin_bit_cast(s16x8, ring[t % kPrefetchK]);
-          if (t % kIssueEvery == 0) fetch_piece(t / kIssueEvery, k1, v1);
+          if (!kSecond && t % kSEvery == 0) fetch_piece(NI + t / kSEvery, kt_k, ts_k, knext);
 #pragma unroll
           for (int mb = 0; mb < MB; ++mb)
             s_acc[mb][t & 1] = E::mfma(ka, qreg[mb][t >> 1], (t >> 1) == 0 ? kZero16 : s_acc[mb][t & 1]);
           if (t + kPrefetchK < 2 * DS) ring[t % kPrefetchK] = read_k(t + kPrefetchK);
           __builtin_amdgcn_sched_barrier(0);
         }
+      } else if (!kSecond) {
+#pragma unroll
+        for (int piece = NI; piece < 2 * NI; ++piece) fetch_piece(piece, kt_k, ts_k, knext);
+      }
 
-        // ---- online softmax, one query per lane ----
-        // Scores are handled as plain scalars (element writes into the MFMA vector types
-        // make the compiler copy whole vectors), P is packed two values per register.
+      if (kSecond) __builtin_amdgcn_s_waitcnt(0x0F70);  // staging step i of this wavefront has landed
+      __builtin_amdgcn_s_barrier();
+      if (kSecond) {
+        // staging step i + 1: K(i + 2) into the buffer of K(i), V(i + 1) into that of V(i - 1)
+#pragma unroll
+        for (int piece = 0; piece < 2 * NI; ++piece)
+          fetch_piece(piece, piece < NI ? kt_k - 1 : kt_k, piece < NI ? ts_v : ts_k,
+                      const_cast<char*>(piece < NI ? vprev : kcur));
+      }
+
+      // ---- X(i): online softmax of tile i, one query per lane ----
+      // Scores are handled as plain scalars (element writes into the MFMA vector types
+      // make the compiler copy whole vectors), P is packed two values per register.
+      if (work_cur) {
+        asm volatile("");
         const bool need_mask = key0 + kTileN > wave_min;
-        s16x8 p_op[MB][4];  // P^T as B operands of the 4 k-steps (16 keys each)
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
           float sc[32];
 #pragma unroll
           for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) sc[kb * 16 + i] = s_acc[mb][kb][i];
+            for (int x = 0; x < 16; ++x) sc[kb * 16 + x] = s_acc[mb][kb][x];
           if (need_mask) {
             asm volatile("");  // keeps this a branch: turned into selects it would run on every tile
-            // register i of block kb is key kb*32 + (i/4)*8 + half*4 + i%4 of the tile
+            // register x of block kb is key kb*32 + (x/4)*8 + half*4 + x%4 of the tile
             const int rel = lim[mb] - key0 - half * 4;
 #pragma unroll
             for (int x = 0; x < 32; ++x) {
@@ -439,57 +542,42 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
           for (int x = 0; x < 32; x += 2) {
             const float p0 = fast_exp2(fmaf(sc[x], a.qscale, -m_safe));
             const float p1 = fast_exp2(fmaf(sc[x + 1], a.qscale, -m_safe));
-            psum += p0 + p1;
             pw[x >> 1] = E::pack2(p0, p1);
+            psum += p0 + p1;
           }
           // k-step j takes registers 8j .. 8j+7 of the 32 scores = words 4j .. 4j+3
 #pragma unroll
           for (int j = 0; j < 4; ++j)
             p_op[mb][j] = __builtin_bit_cast(s16x8, v4u{pw[4 * j], pw[4 * j + 1], pw[4 * j + 2], pw[4 * j + 3]});
-          if (moved) {
-            asm volatile("");  // likewise: the rescale is rare and must not run unconditionally
-            l_run[mb] = l_run[mb] * alpha + psum;
-#pragma unroll
-            for (int db = 0; db < DB; ++db) o_acc[mb][db] *= alpha;
-          } else {
-            l_run[mb] += psum;
-          }
-        }
-
-        // ---- O^T += V^T P^T ----
-        {
-          // step t = (j, db): this lane names the chunk (key = base + bi / 4, d = dblock + 4 * (bi % 4))
-          // and receives d = dblock + bi for keys base .. base + 3, once for each half of the 16 keys
-          auto read_v = [&](int t, s16x4& lo, s16x4& hi) {
-            const int j = t / DB, db = t % DB;
-            const char* p0 = vcur + vofs[db] + ((j >> 1) * 32 + (j & 1) * 16) * ROWB;
-            lo = lds_read_tr(p0);
-            hi = lds_read_tr(p0 + 8 * ROWB);
-          };
-          s16x4 rlo[kPrefetchV], rhi[kPrefetchV];
-#pragma unroll
-          for (int t = 0; t < kPrefetchV; ++t) read_v(t, rlo[t], rhi[t]);
-          __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int t = 0; t < 4 * DB; ++t) {
-            const s16x4 lo = rlo[t % kPrefetchV], hi = rhi[t % kPrefetchV];
-            const s16x8 va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-#pragma unroll
-            for (int mb = 0; mb < MB; ++mb) o_acc[mb][t % DB] = E::mfma(va, p_op[mb][t / DB], o_acc[mb][t % DB]);
-            if (t + kPrefetchV < 4 * DB) read_v(t + kPrefetchV, rlo[t % kPrefetchV], rhi[t % kPrefetchV]);
-            __builtin_amdgcn_sched_barrier(0);
-          }
+          l_run[mb] = fmaf(l_run[mb], alpha, psum);  // alpha is 1 unless the reference point moved
+          // the accumulators are rescaled where they are next used, at the start of M(i + 1)
+          alpha_next[mb] = alpha;
+          moved_next[mb] = moved;
         }
       }
-
-      __builtin_amdgcn_s_waitcnt(0x0F70);  // this wavefront's share of tile kt + 1 has landed
-      __syncthreads();
     };
 
-    for (int kt = 0; kt < n_kv_tiles; kt += 2) {
-      tile_step(IntC<0>{}, kt);
-      if (kt + 1 < n_kv_tiles) tile_step(IntC<1>{}, kt + 1);
+    // steps 0 .. n_kv_tiles (the last one only has the O^T part of the last tile)
+    if (wave < kWaves / 2) {
+      for (int i = 0; i <= n_kv_tiles; i += 2) {
+        step(IntC<0>{}, IntC<0>{}, i);
+        if (i + 1 <= n_kv_tiles) step(IntC<0>{}, IntC<1>{}, i + 1);
+      }
+      __builtin_amdgcn_s_barrier();  // the second half's last barrier
+    } else {
+      __builtin_amdgcn_s_barrier();  // barrier 0: the first half starts M(0)
+      {  // staging step 0: K(1), V(0)
+        const int ts1 = tile_slot(1), ts0 = tile_slot(0);
+#pragma unroll
+        for (int piece = 0; piece < 2 * NI; ++piece)
+          fetch_piece(piece, piece < NI ? 0 : 1, piece < NI ? ts0 : ts1, piece < NI ? s_v0 : s_k1);
+      }
+      for (int i = 0; i <= n_kv_tiles; i += 2) {
+        step(IntC<1>{}, IntC<0>{}, i);
+        if (i + 1 <= n_kv_tiles) step(IntC<1>{}, IntC<1>{}, i + 1);
+      }
     }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // no staging load is in flight when the LDS tiles are reused
 
     // ---- finish the run: normalise and store ----
 #pragma unroll
