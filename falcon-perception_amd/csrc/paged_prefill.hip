@@ -190,11 +190,34 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
   const int bi = lane & 15;
   const int tile0 = tile * BM;
 
-  for (int i = tid; i < BM; i += kThreads) {
-    const int r = tile0 + i;
-    int64_t bx = r < a.Lq ? a.batch_idx[r] : 0;
+  // Everything the set-up needs from global memory is requested at once, so the loads travel
+  // together: the sequence of each row of the tile, then this wavefront's row limits and Q rows.
+  // Rows outside a run keep their Q values: what such a row computes is never stored.
+  int64_t bx_raw[(BM + kThreads - 1) / kThreads];
+#pragma unroll
+  for (int j = 0; j < (BM + kThreads - 1) / kThreads; ++j) {
+    const int r = tile0 + j * kThreads + tid;
+    bx_raw[j] = (j * kThreads + tid < BM && r < a.Lq) ? a.batch_idx[r] : 0;
+  }
+  int row[MB], lim_raw[MB];
+  s16x8 qreg[MB][DS];  // Q^T operands: lane (query ln, half) holds d = 16*ds + 8*half .. +8 for every k-step
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    row[mb] = tile0 + (rblock * MB + mb) * 32 + ln;
+    const bool in = row[mb] < a.Lq;
+    lim_raw[mb] = in ? a.row_limit[row[mb]] : 0;
+#pragma unroll
+    for (int ds = 0; ds < DS; ++ds) {
+      v4u w = {0, 0, 0, 0};
+      if (in) w = *reinterpret_cast<const v4u*>(a.q + row[mb] * a.qs_row + hq * a.qs_h + (16 * ds + 8 * half) * 2);
+      qreg[mb][ds] = __builtin_bit_cast(s16x8, w);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < (BM + kThreads - 1) / kThreads; ++j) {
+    int64_t bx = bx_raw[j];
     if (bx < 0 || bx >= a.max_batch) bx = 0;
-    s_bidx[i] = static_cast<int>(bx);
+    if (j * kThreads + tid < BM) s_bidx[j * kThreads + tid] = static_cast<int>(bx);
   }
   __syncthreads();
 
@@ -219,19 +242,27 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
     // values every lane agrees on are moved to scalar registers so the control flow that
     // depends on them stays uniform
     const int sq = __builtin_amdgcn_readfirstlane(s_bidx[run0]);
-    int run1 = run0 + 1;
-    while (run1 < BM && __builtin_amdgcn_readfirstlane(s_bidx[run1]) == sq) ++run1;
+    // end of the run: the first row of another sequence, found 64 rows at a time
+    int run1 = BM;
+    for (int base = run0; base < BM; base += 64) {
+      const int idx = base + lane;
+      const unsigned long long other = __ballot(idx < BM && s_bidx[idx] != sq);
+      if (other != 0) {
+        run1 = base + __builtin_ctzll(other);
+        break;
+      }
+    }
+    run1 = __builtin_amdgcn_readfirstlane(run1);
 
     // rows of this wavefront: tile rows rblock * 32 + ln
-    int row[MB], lim[MB];
+    int lim[MB];
     bool active[MB];
     int my_max = 0;
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
       const int tr = (rblock * MB + mb) * 32 + ln;
-      row[mb] = tile0 + tr;
       active[mb] = tr >= run0 && tr < run1 && row[mb] < a.Lq;
-      lim[mb] = (active[mb] && sq != 0) ? a.row_limit[row[mb]] : 0;
+      lim[mb] = (active[mb] && sq != 0) ? lim_raw[mb] : 0;
       if (lim[mb] < 0) lim[mb] = 0;
       my_max = max(my_max, lim[mb]);
     }
@@ -271,19 +302,6 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
     for (int w = 0; w < kWaves; ++w) kv_max = max(kv_max, s_red[w]);
     kv_max = __builtin_amdgcn_readfirstlane(kv_max);
     const int n_kv_tiles = (kv_max + kTileN - 1) / kTileN;
-
-    // Q^T operands: lane (query ln, half) holds d = 16*ds + 8*half .. +8 for every k-step
-    s16x8 qreg[MB][DS];
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-#pragma unroll
-      for (int ds = 0; ds < DS; ++ds) {
-        v4u w = {0, 0, 0, 0};
-        if (active[mb])
-          w = *reinterpret_cast<const v4u*>(a.q + row[mb] * a.qs_row + hq * a.qs_h + (16 * ds + 8 * half) * 2);
-        qreg[mb][ds] = __builtin_bit_cast(s16x8, w);
-      }
-    }
 
     f32x16 o_acc[MB][DB];
     float m_run[MB], l_run[MB];

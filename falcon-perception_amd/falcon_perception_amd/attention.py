@@ -124,11 +124,18 @@ class HybridPrefillMask:
         self.seq_lengths = (L, L)
         self.row_hi = ops.hybrid_row_limits(input_ids, soi_id, eoi_id)  # [L] int32, packed coordinates
         self._arange = torch.arange(L, dtype=torch.int64, device=batch_idx.device)
+        self._step_key = None  # the step whose row limits are kept below
+        self._row_limit = None
 
     def row_limit(self, input_pos: Tensor) -> Tensor:
-        """Logical key limit of each row: its position plus the reach of `row_hi` beyond the row."""
-        reach = self.row_hi.to(torch.int64) - self._arange
-        return (input_pos.reshape(-1) + reach).to(torch.int32)
+        """Logical key limit of each row: its position plus the reach of `row_hi` beyond the row.
+        Computed by the first layer of a step and kept for the others."""
+        key = (input_pos.data_ptr(), input_pos._version, tuple(input_pos.shape))
+        if key != self._step_key:
+            reach = self.row_hi.to(torch.int64) - self._arange
+            self._row_limit = (input_pos.reshape(-1) + reach).to(torch.int32)
+            self._step_key = key
+        return self._row_limit
 
 
 # --------------------------------------------------------------------------
