@@ -504,13 +504,67 @@ template <typename E, int D>
 __global__ __launch_bounds__(64) void paged_decode_merge_kernel(const DecodeArgs a) {
   const int hq = blockIdx.x;
   const int b = blockIdx.y;
+  const int64_t p0 = (static_cast<int64_t>(b) * a.Hq + hq) * a.n_splits;
+
+  // The kernel is a chain of memory latencies, so when the launch has at most kBatch splits every
+  // load is requested at once, the partials of splits this sequence does not have included (they are
+  // dropped by a select once its length is known, never used in arithmetic).
+  constexpr int kBatch = 8;
+  constexpr int DPL = (D + 63) / 64;  // output elements per lane
+  const bool batched = a.n_splits <= kBatch;
+  float m_s[kBatch], l_s[kBatch], acc_s[kBatch][DPL];
+  if (batched) {
+#pragma unroll
+    for (int s = 0; s < kBatch; ++s) {
+      const bool on = s < a.n_splits;
+      m_s[s] = on ? a.ws_ml[(p0 + s) * 2] : -INFINITY;
+      l_s[s] = on ? a.ws_ml[(p0 + s) * 2 + 1] : 0.f;
+#pragma unroll
+      for (int j = 0; j < DPL; ++j) {
+        const int d = threadIdx.x + j * 64;
+        acc_s[s][j] = (on && d < D) ? a.ws_acc[(p0 + s) * D + d] : 0.f;
+      }
+    }
+  }
+
   int64_t L = fp::load_index(a.input_pos, b, a.pos_i64) + 1;
   const int64_t trow = a.batch_idx[b];
   if (trow < 0 || trow >= a.max_batch) L = 0;
   if (L > a.max_context) L = a.max_context;
   const int part = split_part(static_cast<int>(L), a.split_tokens);
   const int ns = L <= 0 ? 0 : static_cast<int>((L + part - 1) / part);
-  const int64_t p0 = (static_cast<int64_t>(b) * a.Hq + hq) * a.n_splits;
+
+  if (batched) {
+    float mn = -INFINITY;
+#pragma unroll
+    for (int s = 0; s < kBatch; ++s) {
+      if (s >= ns) m_s[s] = -INFINITY;
+      mn = fmaxf(mn, m_s[s]);
+    }
+    const float ms = safe_max(mn);
+    float den = 0.f, num[DPL];
+#pragma unroll
+    for (int j = 0; j < DPL; ++j) num[j] = 0.f;
+#pragma unroll
+    for (int s = 0; s < kBatch; ++s) {
+      if (s < ns) {  // same order of additions as the loops below
+        const float wgt = fast_exp2(m_s[s] - ms);
+        den += l_s[s] * wgt;
+#pragma unroll
+        for (int j = 0; j < DPL; ++j) num[j] += acc_s[s][j] * wgt;
+      }
+    }
+    const float lse_nat = ns > 0 ? (mn + log2f(den)) * kLn2 : -INFINITY;
+#pragma unroll
+    for (int j = 0; j < DPL; ++j) {
+      const int d = threadIdx.x + j * 64;
+      if (d >= D) continue;
+      const float o = ns > 0 ? num[j] / den : 0.f;
+      E::store(a.out + b * a.os_b + hq * a.os_h + d * sizeof(typename E::type), sink_gate<E>(o, lse_nat, a.sinks, hq));
+    }
+    if (threadIdx.x == 0) a.lse[static_cast<int64_t>(b) * a.Hq + hq] = lse_nat;
+    return;
+  }
 
   float mn = -INFINITY;
   for (int s = 0; s < ns; ++s) mn = fmaxf(mn, a.ws_ml[(p0 + s) * 2]);
