@@ -431,6 +431,14 @@ def append_gather_rates(steps: int = 20, T: int = 32768, H: int = 16, D: int = 1
     e = 2
     bytes_a = 2 * T * (2 * H * D * e) + 8 * T
     bytes_g = 2 * T * (H * D * e)
+    # the same append over the first t tokens, from a decode step's worth of rows up to the whole batch
+    sweep = {}
+    for t in (64, 512, 4096, T):
+        def do_part(t=t):
+            ops.kv_append(pk, pv, k_rows[:t], v_rows[:t], cache.page_table, flat_b[:t], flat_p[:t], P,
+                          clamp_negative=False)
+        ms_t = event_ms(do_part, steps)
+        sweep[str(t)] = {"ms": ms_t, "gbps": (2 * t * (2 * H * D * e) + 8 * t) / (ms_t * 1e-3) / 1e9}
 
     # QK norm + rotary embedding + insert in one launch (reference model.py:110-119 + the append):
     # the qkv projection output of the same step, 16 query heads / 8 kv heads, expanded to the 16 cached heads
@@ -459,6 +467,7 @@ def append_gather_rates(steps: int = 20, T: int = 32768, H: int = 16, D: int = 1
             "qkv_norm_rope_append_frac_of_peak": bytes_r / (ms_r * 1e-3) / 1e9 / HBM_PEAK_GBPS,
             "kv_append_ms": ms_a, "kv_append_gbps": bytes_a / (ms_a * 1e-3) / 1e9,
             "kv_append_frac_of_peak": bytes_a / (ms_a * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "kv_append_by_tokens": sweep,
             "kv_gather_ms": ms_g, "kv_gather_gbps": bytes_g / (ms_g * 1e-3) / 1e9,
             "kv_gather_frac_of_peak": bytes_g / (ms_g * 1e-3) / 1e9 / HBM_PEAK_GBPS}
 
