@@ -15,10 +15,13 @@
 //         (plus one exchange between the two lane halves).
 //   O^T = V^T P^T: P^T is already in B-operand layout in the S^T accumulators; V^T
 //         comes out of LDS through ds_read_b64_tr_b16, so V is staged row-major like K.
-//   K/V tiles of 64 keys are fetched page by page one tile ahead with global_load_lds
-//   (16 bytes per lane straight into LDS, no staging registers), page ids two tiles ahead
-//   and turned into row addresses right after the barrier, into a double buffer whose rows
-//   are chunk-permuted against bank conflicts.
+//   K/V tiles of 64 keys go straight from global memory into LDS with global_load_lds
+//   (16 bytes per lane, no staging registers), into double buffers whose rows are
+//   chunk-permuted against bank conflicts; the first pool slot of every tile of a run is
+//   looked up once, so a staging load is a scalar base plus a fixed lane offset.
+//   The two wavefronts that share a SIMD run half a step apart (two barriers per tile): one is
+//   in its MFMA phase (O^T of the previous tile, S^T of the current one) while the other is in
+//   its softmax.
 // Rows of one tile may belong to several sequences: the tile is processed one
 // run of equal batch_idx at a time; rows of slot 0 are padding (out 0, lse -inf).
 #include "fp_common.h"
@@ -392,13 +395,14 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
     // ---- schedule ----
     // Step i of a wavefront is M(i) = { O^T += V^T P^T of tile i - 1;  S^T = K Q^T of tile i } on the
     // matrix pipe, then X(i) = softmax of tile i on the vector pipe.  The two wavefronts that share a
-    // SIMD (w and w + 4) run half a step apart, held there by two barriers per step: while one is in
-    // M the other is in X, so the matrix and the vector pipe of the SIMD work at the same time.
-    //   barrier 2i     first half: M(i)     second half: X(i - 1)
-    //   barrier 2i+1   first half: X(i)     second half: M(i)
-    // Staging step i (K of tile i + 1, V of tile i) is issued after barrier 2i, when M(i - 1) is over
-    // everywhere, and has landed before barrier 2i + 2, after which M(i + 1) begins.  K(i) lives in
-    // K buffer i % 2, V(i) in V buffer i % 2.
+    // SIMD (w and w + 4) run half a step apart: between two barriers the first half does M(i) then
+    // X(i), the second half X(i - 1) then M(i), so that one is in M while the other is in X and the
+    // matrix and the vector pipe of the SIMD work at the same time.  One barrier per step (B(i), at the
+    // start of the first half's step and in the middle of the second half's) is all the data needs:
+    // staging step i (K of tile i + 1, V of tile i) is issued after B(i), when M(i - 1) is over
+    // everywhere, and every wavefront has waited for its loads before B(i + 1), after which M(i + 1)
+    // begins.  (A second barrier between the two parts of the interval kept the halves in step more
+    // strictly and cost 2 %.)  K(i) lives in K buffer i % 2, V(i) in V buffer i % 2.
     {
       const int ts0 = tile_slot(0);
 #pragma unroll
@@ -436,7 +440,7 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
       const int ts_k = tile_slot(kt_k);
       const int ts_v = tile_slot(kt_k - 1);
       if (!kSecond) __builtin_amdgcn_s_waitcnt(0x0F70);  // staging step i - 1 of this wavefront has landed
-      __builtin_amdgcn_s_barrier();
+      if (!kSecond) __builtin_amdgcn_s_barrier();
 
       // ---- M(i), first part: O^T += V^T P^T of tile i - 1 ----
       f32x16 s_acc[MB][2];  // written by the first MFMA of each block, which starts from zero
@@ -509,7 +513,7 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
       }
 
       if (kSecond) __builtin_amdgcn_s_waitcnt(0x0F70);  // staging step i of this wavefront has landed
-      __builtin_amdgcn_s_barrier();
+      if (kSecond) __builtin_amdgcn_s_barrier();
       if (kSecond) {
         // staging step i + 1: K(i + 2) into the buffer of K(i), V(i + 1) into that of V(i - 1)
 #pragma unroll
@@ -581,9 +585,9 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
         step(IntC<0>{}, IntC<0>{}, i);
         if (i + 1 <= n_kv_tiles) step(IntC<0>{}, IntC<1>{}, i + 1);
       }
-      __builtin_amdgcn_s_barrier();  // the second half's last barrier
+      __builtin_amdgcn_s_barrier();  // the second half's last barrier, B(n_kv_tiles + 1)
     } else {
-      __builtin_amdgcn_s_barrier();  // barrier 0: the first half starts M(0)
+      __builtin_amdgcn_s_barrier();  // B(0): the first half starts M(0)
       {  // staging step 0: K(1), V(0)
         const int ts1 = tile_slot(1), ts0 = tile_slot(0);
 #pragma unroll
