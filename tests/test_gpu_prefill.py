@@ -183,3 +183,23 @@ def test_fp32_rows_over_a_context_longer_than_the_page_list():
     assert_close(out, lse, eo, el, dtype)
     assert not f64(out)[:, :, :2].any() and np.isneginf(f64(lse)[:, :, :2]).all()
     assert lse.shape == (1, 2, len(lims))
+
+
+def test_a_run_longer_than_the_tile_slot_table():
+    """The MFMA kernel looks up the first pool slot of up to 2048 tiles (131072 keys) of a run ahead of its
+    tile loop; the tiles beyond, like the last tile of any run, are staged row by row.  Limits on both sides
+    of that boundary, one of them ending inside a tile."""
+    dtype, P, D = torch.bfloat16, 128, 64
+    L = 2048 * 64 + 300
+    st = PagedState(11, n_pages=L // P + 8, page_size=P, max_batch=3, Hc=1, D=D, dtype=dtype)
+    b = st.add_sequence(L)
+    st.prefill_random()
+    lims = [2048 * 64 - 1, 2048 * 64, 2048 * 64 + 1, 2048 * 64 + 64, 2048 * 64 + 150, L]
+    q = randn(st.gen, (1, 2, len(lims), D), dtype)
+    bidx = torch.full((len(lims),), b, dtype=torch.int64)
+    lim = torch.tensor(lims, dtype=torch.int32)
+    pk, pv = st.pool_planes()
+    out, lse = ops.paged_prefill(q.to(DEV), pk, pv, st.cache.page_table, bidx.to(DEV), lim.to(DEV), P)
+    eo, el = O.prefill_attention_paged(f64(q), f64(pk), f64(pv), st.mirror.page_table, bidx.numpy(),
+                                       None, lim.numpy(), P)
+    assert_close(out, lse, eo, el, dtype)
