@@ -31,6 +31,7 @@ import torch  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, published peak
+MFMA_F32_PEAK_TFLOPS = 157.3    # MI355X dense fp32 MFMA, published peak
 MODEL_LAYERS = 28       # Falcon Perception 0.6B (reference __init__.py:36)
 
 # name -> shape of the decode workloads of BASELINE.json (configs[0], [1], [3] decode part, [4])
@@ -204,6 +205,8 @@ PREFILL_WORKLOADS = {
     # whole sequences in one step (prefix 0): the image span rows are bidirectional
     "cfg3w": dict(seed=3, dtype="bf16", n_seq=8, Hq=16, Hc=8, D=128, P=128, prefix_lo=256, prefix_hi=4096, chunk=512,
                   whole=True),
+    # cfg3 in the reference's default dtype (reference server/config.py:38)
+    "cfg3f32": dict(seed=3, dtype="f32", n_seq=8, Hq=16, Hc=8, D=128, P=128, prefix_lo=256, prefix_hi=4096, chunk=512),
 }
 
 
@@ -483,10 +486,15 @@ def prefill_rate(steps: int = 10, name: str = "cfg3") -> dict:
     tf = case.flops() / (ms * 1e-3) / 1e12
     what = {"cfg3": "cfg3: 8 sequences, paged prefix U[256,4096], 512-token chunk each, 16 q / 8 kv heads, D 128",
             "cfg3w": "cfg3w: the same 8 sequences prefilled whole (prefix + chunk rows in one step, prefix rows see "
-                     "their whole image span), 16 q / 8 kv heads, D 128"}[name]
-    return {"workload": what, "query_rows": int(case.q.shape[2]),
-            "paged_prefill_ms": ms, "tflops": tf, "frac_of_bf16_mfma_peak": tf / MFMA_BF16_PEAK_TFLOPS,
-            "chunk_append_ms": ms_a, "flops": case.flops()}
+                     "their whole image span), 16 q / 8 kv heads, D 128",
+            "cfg3f32": "cfg3 in fp32"}[name]
+    res = {"workload": what, "query_rows": int(case.q.shape[2]), "paged_prefill_ms": ms, "tflops": tf,
+           "chunk_append_ms": ms_a, "flops": case.flops()}
+    if case.q.dtype == torch.float32:
+        res["frac_of_f32_mfma_peak"] = tf / MFMA_F32_PEAK_TFLOPS
+    else:
+        res["frac_of_bf16_mfma_peak"] = tf / MFMA_BF16_PEAK_TFLOPS
+    return res
 
 
 def cpu_baseline(case: DecodeCase, budget_s: float = 20.0) -> dict:
@@ -622,6 +630,7 @@ def main() -> int:
     if not args.decode_only:
         result["prefill_sized"] = append_gather_rates()
         result["chunked_prefill"] = prefill_rate()
+        result["chunked_prefill_fp32"] = prefill_rate(name="cfg3f32")
         ms_model = model_depth_graph_ms(case, args.steps)  # last: it takes and returns 56 GiB
         if ms_model is not None:
             result["ms_all_layers_hip_graph"] = ms_model

@@ -54,8 +54,8 @@ struct PageDiv {
   }
 };
 
-// fp32 chunked-prefill attention, served by the single-query kernel in row mode (paged_decode.hip)
-int prefill_rows_f32(const void* q, int64_t q_stride_row, int64_t q_stride_h, const void* pool_k, const void* pool_v,
+// fp32 chunked-prefill attention on the fp32 matrix instruction (paged_prefill_f32.hip)
+int prefill_mfma_f32(const void* q, int64_t q_stride_row, int64_t q_stride_h, const void* pool_k, const void* pool_v,
                      const int64_t* page_table, int64_t pt_row_stride, const int64_t* batch_idx,
                      const int32_t* row_limit, void* out, int64_t out_stride_row, int64_t out_stride_h, float* lse,
                      const float* sinks, int32_t Lq, int32_t Hq, int32_t Hc, int32_t D, int32_t page_size,

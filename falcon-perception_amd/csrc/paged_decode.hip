@@ -45,7 +45,6 @@ struct DecodeArgs {
   char* out;
   int64_t os_b, os_h;  // bytes
   float* lse;
-  int64_t lse_sh;  // row mode only: lse is [Hq, rows] with this head stride
   const float* sinks;  // optional [Hq]: out is multiplied by sigmoid(lse - sinks[h])
   float* ws_acc;  // [B, Hq, n_splits, D]
   float* ws_ml;   // [B, Hq, n_splits, 2]
@@ -258,18 +257,13 @@ __device__ __forceinline__ void fold_rows(const v4u (&kreg)[GK][U], const v4u (&
 // kAligned: the page size is a power of two and a multiple of the rows one
 // wavefront iteration covers, so those rows share one page and one base address.
 //
-// kRowMode serves chunked-prefill attention in fp32 through the same code: every packed query row is
-// a "sequence" of its own (grid y = row), input_pos holds the row's key limit (not limit - 1), rows
-// of cache slot 0 are padding, lse is [Hq, rows], and the one split of a row may span more pages
-// than the LDS page list holds, so the list is refilled every 512 pages.
-//
 // kPerHeadK serves a cache that holds one K head per QUERY head (the reference stores K and V
 // expanded to n_heads because the 2D rotary angles differ per head, model.py:112-114) whose V heads
 // are n_rep identical copies: a workgroup takes the G = n_rep query heads of one group, reads their G
 // K rows and ONE V row (the first copy), i.e. (G + 1) / 2G of the bytes an expanded read costs.
 constexpr int decode_loads_in_flight(int G, bool per_head_k) { return per_head_k && G >= 4 ? 4 : 8; }
 
-template <typename E, int D, int G, bool kDirect, bool kAligned, bool kRowMode = false, bool kPerHeadK = false>
+template <typename E, int D, int G, bool kDirect, bool kAligned, bool kPerHeadK = false>
 __global__ __launch_bounds__(kThreads) void paged_decode_kernel(const DecodeArgs a) {
   constexpr int EPL = E::kEpl;          // elements per lane
   constexpr int TPR = D / EPL;          // lanes per row
@@ -295,12 +289,12 @@ __global__ __launch_bounds__(kThreads) void paged_decode_kernel(const DecodeArgs
   const int grp = lane / TPR;  // row of this lane inside a wavefront load
   const int col = lane % TPR;  // 16-byte chunk of the row
 
-  int64_t L = fp::load_index(a.input_pos, b, a.pos_i64) + (kRowMode ? 0 : 1);
+  int64_t L = fp::load_index(a.input_pos, b, a.pos_i64) + 1;
   const int64_t trow = a.batch_idx[b];
-  if (trow < 0 || trow >= a.max_batch || (kRowMode && trow == 0)) L = 0;
+  if (trow < 0 || trow >= a.max_batch) L = 0;
   if (L > a.max_context) L = a.max_context;
   auto lse_at = [&](int hq) -> float& {
-    return a.lse[kRowMode ? hq * a.lse_sh + b : static_cast<int64_t>(b) * a.Hq + hq];
+    return a.lse[static_cast<int64_t>(b) * a.Hq + hq];
   };
   // A context of L tokens is cut into ceil(L / split_tokens) parts of equal size (a multiple of
   // 64 tokens), so the workgroups of one sequence carry the same load instead of leaving a short
@@ -346,30 +340,26 @@ __global__ __launch_bounds__(kThreads) void paged_decode_kernel(const DecodeArgs
   const char* kbase = a.pool_k + static_cast<int64_t>(kPerHeadK ? hc * G : hc) * head_stride + col * 16;
   const char* vbase = a.pool_v + static_cast<int64_t>(kPerHeadK ? hc * G : hc) * head_stride + col * 16;
 
-  // page ids of the split -> LDS, then the rows.  Outside row mode one round covers the split.
+  // page ids of the split -> LDS, then the rows
   int64_t blk0;
-  int s0 = t0;
-  while (true) {
-    const int span = 512 * a.pd.page_size;  // a multiple of the page size and of kWaves * CH
-    const int s1 = (kRowMode && t1 - s0 > span) ? s0 + span : t1;
-    {
-      int off_unused;
-      a.pd.split(s0, blk0, off_unused);
-      int64_t blk_last;
-      a.pd.split(s1 - 1, blk_last, off_unused);
-      const int nblk = static_cast<int>(blk_last - blk0) + 1;
-      for (int i = tid; i < nblk; i += kThreads) {
-        int64_t page = 0;
-        if (blk0 + i < a.n_pages) page = a.page_table[trow * a.pt_row_stride + blk0 + i];
-        if (page < 0 || page >= a.n_slots / a.pd.page_size) page = 0;  // not a page of the pool
-        s_pages[i] = static_cast<int>(page);
-      }
+  {
+    int off_unused;
+    a.pd.split(t0, blk0, off_unused);
+    int64_t blk_last;
+    a.pd.split(t1 - 1, blk_last, off_unused);
+    const int nblk = static_cast<int>(blk_last - blk0) + 1;
+    for (int i = tid; i < nblk; i += kThreads) {
+      int64_t page = 0;
+      if (blk0 + i < a.n_pages) page = a.page_table[trow * a.pt_row_stride + blk0 + i];
+      if (page < 0 || page >= a.n_slots / a.pd.page_size) page = 0;  // not a page of the pool
+      s_pages[i] = static_cast<int>(page);
     }
-    __syncthreads();
-    const int c_end = t1_pool < s1 ? t1_pool : s1;
+  }
+  __syncthreads();
+  const int c_end = t1_pool;
 
 #pragma nounroll
-  for (int c0 = s0 + wave * CH; c0 < c_end; c0 += kWaves * CH) {
+  for (int c0 = t0 + wave * CH; c0 < c_end; c0 += kWaves * CH) {
     v4u kreg[GK][U], vreg[U];
     if (kAligned) {
       // the CH rows of this iteration lie in one page: one base, constant offsets
@@ -401,10 +391,6 @@ __global__ __launch_bounds__(kThreads) void paged_decode_kernel(const DecodeArgs
       fold_rows<E, TPR, G, GK, U, RPW, false>(kreg, vreg, q, a.qscale, c0 + grp, c_end, m, l, acc);
     else
       fold_rows<E, TPR, G, GK, U, RPW, true>(kreg, vreg, q, a.qscale, c0 + grp, c_end, m, l, acc);
-  }
-    if (!kRowMode || s1 >= t1) break;
-    __syncthreads();  // every wavefront is done with the page list before it is refilled
-    s0 = s1;
   }
 
   if (t1_pool != t1 && wave == 0) {
@@ -595,15 +581,15 @@ void launch_decode(const DecodeArgs& a, int B, int phases, hipStream_t st) {
     // one split covers every context: the partial pass writes out and lse itself
     if (!(phases & kPhasePartial)) return;
     if (aligned)
-      hipLaunchKernelGGL((paged_decode_kernel<E, D, G, true, true, false, kPerHeadK>), grid, dim3(kThreads), 0, st, a);
+      hipLaunchKernelGGL((paged_decode_kernel<E, D, G, true, true, kPerHeadK>), grid, dim3(kThreads), 0, st, a);
     else
-      hipLaunchKernelGGL((paged_decode_kernel<E, D, G, true, false, false, kPerHeadK>), grid, dim3(kThreads), 0, st, a);
+      hipLaunchKernelGGL((paged_decode_kernel<E, D, G, true, false, kPerHeadK>), grid, dim3(kThreads), 0, st, a);
   } else {
     if (phases & kPhasePartial) {
       if (aligned)
-        hipLaunchKernelGGL((paged_decode_kernel<E, D, G, false, true, false, kPerHeadK>), grid, dim3(kThreads), 0, st, a);
+        hipLaunchKernelGGL((paged_decode_kernel<E, D, G, false, true, kPerHeadK>), grid, dim3(kThreads), 0, st, a);
       else
-        hipLaunchKernelGGL((paged_decode_kernel<E, D, G, false, false, false, kPerHeadK>), grid, dim3(kThreads), 0, st, a);
+        hipLaunchKernelGGL((paged_decode_kernel<E, D, G, false, false, kPerHeadK>), grid, dim3(kThreads), 0, st, a);
     }
     if (phases & kPhaseMerge)
       hipLaunchKernelGGL((paged_decode_merge_kernel<E, D>), dim3(a.Hq, B), dim3(64), 0, st, a);
@@ -634,28 +620,6 @@ int dispatch_dim(const DecodeArgs& a, int B, int D, int phases, int kv_rep, hipS
     case 64: return dispatch_group<E, 64>(a, B, phases, kv_rep, st);
     case 128: return dispatch_group<E, 128>(a, B, phases, kv_rep, st);
     default: return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_decode: head_dim %d (supported: 64, 128)", D);
-  }
-}
-
-// Row mode (fp32 chunked prefill): one workgroup per (cache head, query row), one split.
-template <int D, int G>
-void launch_rows(const DecodeArgs& a, int rows, hipStream_t st) {
-  dim3 grid(a.Hc, rows, 1);
-  const int chunk_rows = 8 * 64 / (D * 4 / 16);
-  if (a.pd.shift >= 0 && a.pd.page_size % chunk_rows == 0)
-    hipLaunchKernelGGL((paged_decode_kernel<F32, D, G, true, true, true>), grid, dim3(kThreads), 0, st, a);
-  else
-    hipLaunchKernelGGL((paged_decode_kernel<F32, D, G, true, false, true>), grid, dim3(kThreads), 0, st, a);
-}
-
-template <int D>
-int dispatch_rows(const DecodeArgs& a, int rows, hipStream_t st) {
-  switch (a.Hq / a.Hc) {
-    case 1: launch_rows<D, 1>(a, rows, st); return FP_OK;
-    case 2: launch_rows<D, 2>(a, rows, st); return FP_OK;
-    case 4: launch_rows<D, 4>(a, rows, st); return FP_OK;
-    case 8: launch_rows<D, 8>(a, rows, st); return FP_OK;
-    default: return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill: Hq/Hc = %d (supported: 1, 2, 4, 8)", a.Hq / a.Hc);
   }
 }
 
@@ -746,7 +710,7 @@ int decode_entry(int phases, const NewRows* fresh, const void* q, int64_t q_stri
   DecodeArgs a{static_cast<const char*>(q), q_stride_b * eb, q_stride_h * eb,
                static_cast<const char*>(pool_k), static_cast<const char*>(pool_v),
                page_table, pt_row_stride, batch_idx, input_pos, pos_index_type == FP_INDEX_I64,
-               static_cast<char*>(out), out_stride_b * eb, out_stride_h * eb, lse, 0, sinks,
+               static_cast<char*>(out), out_stride_b * eb, out_stride_h * eb, lse, sinks,
                nullptr, nullptr, Hq, wg_heads, fp::PageDiv(page_size), n_pages, max_batch, n_slots,
                max_context, split_tokens, ns, scale * kLog2e,  // scores are kept in log2 units
                nullptr, nullptr, 0, 0, 0, 0};
@@ -809,26 +773,3 @@ extern "C" int fp_paged_decode_append(const void* k_new, const void* v_new, int6
   return decode_entry(kPhasePartial | kPhaseMerge, &fresh, FP_DECODE_ARGS);
 }
 
-
-// fp32 chunked-prefill attention: every query row goes through the single-query kernel as a
-// sequence of its own (bandwidth-bound: K/V of a sequence are re-read per row, mostly from L2).
-// Arguments as fp_paged_prefill, already validated there.
-int fp::prefill_rows_f32(const void* q, int64_t q_stride_row, int64_t q_stride_h, const void* pool_k,
-                         const void* pool_v, const int64_t* page_table, int64_t pt_row_stride,
-                         const int64_t* batch_idx, const int32_t* row_limit, void* out, int64_t out_stride_row,
-                         int64_t out_stride_h, float* lse, const float* sinks, int32_t Lq, int32_t Hq, int32_t Hc,
-                         int32_t D, int32_t page_size, int32_t n_pages, int32_t max_batch, int64_t n_slots,
-                         float scale, hipStream_t st) {
-  if (Lq > 65535) return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill: more than 65535 fp32 query rows in one call");
-  constexpr int kNoLimit = 1 << 30;  // one split per row whatever its key limit
-  DecodeArgs a{static_cast<const char*>(q), q_stride_row * 4, q_stride_h * 4,
-               static_cast<const char*>(pool_k), static_cast<const char*>(pool_v),
-               page_table, pt_row_stride, batch_idx, row_limit, 0,
-               static_cast<char*>(out), out_stride_row * 4, out_stride_h * 4, lse, Lq, sinks,
-               nullptr, nullptr, Hq, Hc, fp::PageDiv(page_size), n_pages, max_batch, n_slots,
-               kNoLimit, kNoLimit, 1, scale * kLog2e,
-               nullptr, nullptr, 0, 0, 0, 0};
-  if (D == 64) return dispatch_rows<64>(a, Lq, st);
-  if (D == 128) return dispatch_rows<128>(a, Lq, st);
-  return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill: head_dim %d (supported: 64, 128)", D);
-}

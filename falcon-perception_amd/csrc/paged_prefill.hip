@@ -25,6 +25,7 @@
 // Rows of one tile may belong to several sequences: the tile is processed one
 // run of equal batch_idx at a time; rows of slot 0 are padding (out 0, lse -inf).
 #include "fp_common.h"
+#include "lds_dma.h"
 
 #include <hip/hip_bf16.h>
 #include <hip/hip_fp16.h>
@@ -116,23 +117,7 @@ struct IntC {
   static constexpr int value = N;
 };
 
-// 16 bytes per lane from global memory straight into LDS at `lds` + lane * 16 (`lds` wavefront-uniform).
-// Written as inline assembly on purpose: while the compiler knows of such a load in flight it turns
-// every wait for an LDS read into a wait for all of them, which serialises the operand reads of the
-// main loop against the MFMAs.  The code that issues these loads waits for them itself (vmcnt(0)
-// before the barrier that publishes a tile).
-__device__ __forceinline__ void load_to_lds(const char* src, char* lds) {
-  const uint32_t base = __builtin_amdgcn_readfirstlane(
-      static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds)));
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(base), "v"(src) : "memory");
-}
-
-// The same with the address split into a wavefront-uniform base (scalar registers) and a 32-bit offset per lane.
-__device__ __forceinline__ void load_to_lds(const char* base, uint32_t offset, char* lds) {
-  const uint32_t m0v = __builtin_amdgcn_readfirstlane(
-      static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds)));
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(m0v), "v"(offset), "s"(base) : "memory");
-}
+using fp::load_to_lds;
 
 // K/V tiles in LDS are 64 unpadded rows of D * 2 bytes, filled by global_load_lds (each lane's
 // 16 bytes land at base + lane * 16).  Bank conflicts are avoided by permuting the 16-byte chunks
@@ -677,11 +662,11 @@ extern "C" int fp_paged_prefill(const void* q, int64_t q_stride_row, int64_t q_s
   if (!q || !pool_k || !pool_v || !page_table || !batch_idx || !row_limit || !out || !lse)
     return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_prefill: null pointer");
   if (dtype == FP_DTYPE_F32) {
-    // no fp32 MFMA kernel: the rows go through the single-query kernel, one row per workgroup
+    // fp32 has a kernel of its own on the fp32 matrix instruction
     if (!fp::aligned(q, 16) || !fp::aligned(pool_k, 16) || !fp::aligned(pool_v, 16) || !fp::aligned(out, 4) ||
         (q_stride_row * 4) % 16 || (q_stride_h * 4) % 16)
       return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_prefill: q rows must be 16-byte aligned");
-    const int rc32 = fp::prefill_rows_f32(q, q_stride_row, q_stride_h, pool_k, pool_v, page_table, pt_row_stride, batch_idx,
+    const int rc32 = fp::prefill_mfma_f32(q, q_stride_row, q_stride_h, pool_k, pool_v, page_table, pt_row_stride, batch_idx,
                                           row_limit, out, out_stride_row, out_stride_h, lse, sinks, Lq, Hq, Hc, D, page_size,
                                           n_pages, max_batch, n_slots, scale, static_cast<hipStream_t>(stream));
     if (rc32 != FP_OK) return rc32;

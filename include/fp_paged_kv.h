@@ -300,8 +300,8 @@ int fp_hybrid_row_limits(const int64_t* input_ids, int32_t L,
                          int32_t* row_hi, void* stream);
 
 /*
- * Chunked-prefill attention over the paged cache under the hybrid mask (bf16/f16 on MFMA; fp32
- * rows are served one by one by the single-query kernel).
+ * Chunked-prefill attention over the paged cache under the hybrid mask, on the matrix
+ * instructions of the dtype (bf16, f16, fp32).
  * Replaces compiled_flex_attn_prefill (attention.py:18) as called at model.py:156-162,
  * extended to read the prefix from pages (the reference attends over the packed
  * fresh K/V only, paged_attention.py:393).

@@ -164,9 +164,9 @@ def test_cfg3_chunked_prefill_shape():
         assert_close(out[:, :, rows], lse[:, :, rows], eo, el, torch.bfloat16)
 
 
-def test_fp32_rows_over_a_context_longer_than_the_page_list():
-    """fp32 (the reference's default dtype) has no MFMA kernel: rows go through the single-query kernel,
-    whose LDS page list holds 512 pages per round.  Limits on both sides of that boundary, page size 16."""
+def test_fp32_rows_over_a_long_context_with_small_pages():
+    """fp32 (the reference's default dtype) on its own MFMA kernel: page size 16 is smaller than the
+    kernel's 32-key tile, so every tile is staged row by row; limits around 8192 and a padding row."""
     dtype, P, D = torch.float32, 16, 64
     st = PagedState(9, n_pages=640, page_size=P, max_batch=3, Hc=1, D=D, dtype=dtype)
     b = st.add_sequence(9000)
