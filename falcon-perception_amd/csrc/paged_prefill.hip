@@ -530,9 +530,11 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
               sc[x] = key < rel ? sc[x] : -INFINITY;
             }
           }
-          float mx = sc[0];
+          // four independent chains: one wavefront alone issues a dependent instruction every ~8 cycles
+          float mx4[4] = {sc[0], sc[1], sc[2], sc[3]};
 #pragma unroll
-          for (int x = 1; x < 32; ++x) mx = fmaxf(mx, sc[x]);
+          for (int x = 4; x < 32; ++x) mx4[x & 3] = fmaxf(mx4[x & 3], sc[x]);
+          float mx = fmaxf(fmaxf(mx4[0], mx4[1]), fmaxf(mx4[2], mx4[3]));
           mx = fmaxf(mx, __shfl_xor(mx, 32));
           // Lazy running maximum: the reference point m_run only moves when some row's maximum has
           // grown by more than kMaxSlack (log2 units); until then exp2(s - m_run) may reach
@@ -543,15 +545,19 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
           const float m_safe = m_new == -INFINITY ? 0.f : m_new;
           const float alpha = moved ? fast_exp2(m_run[mb] - m_safe) : 1.f;
           m_run[mb] = m_new;
-          float psum = 0.f;
+          // Stage by stage (scale, exponential, pack and sum) with scheduling barriers between: left alone,
+          // the compiler pairs every exponential with the multiply-add right before it, and a wavefront
+          // that runs alone on the vector pipe waits out the latency of each pair.
+          float part[4] = {0.f, 0.f, 0.f, 0.f};
           uint32_t pw[16];
 #pragma unroll
           for (int x = 0; x < 32; x += 2) {
             const float p0 = fast_exp2(fmaf(sc[x], a.qscale, -m_safe));
             const float p1 = fast_exp2(fmaf(sc[x + 1], a.qscale, -m_safe));
             pw[x >> 1] = E::pack2(p0, p1);
-            psum += p0 + p1;
+            part[(x >> 1) & 3] += p0 + p1;
           }
+          const float psum = (part[0] + part[1]) + (part[2] + part[3]);
           // k-step j takes registers 8j .. 8j+7 of the 32 scores = words 4j .. 4j+3
 #pragma unroll
           for (int j = 0; j < 4; ++j)
