@@ -25,5 +25,16 @@ __device__ __forceinline__ void load_to_lds(const char* base, uint32_t offset, c
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(m0v), "v"(offset), "s"(base) : "memory");
 }
 
+// max(x of lane l, x of lane l ^ 32) in both lanes, without the trip through LDS a shuffle takes:
+// v_permlane32_swap exchanges the upper half of its first operand with the lower half of its second, so
+// from (x, x) it leaves the lower halves' values in one register and the upper halves' in the other.
+// (Inline assembly: the compiler's builtin returned the first register for both results.)  The no-ops
+// cover the wait states between a vector write, the swap and the next vector read.
+__device__ __forceinline__ float max_across_lane_halves(float x) {
+  float lo = x, hi = x;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(lo), "+v"(hi));
+  return fmaxf(lo, hi);
+}
+
 }  // namespace fp
 #endif

@@ -535,7 +535,7 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
 #pragma unroll
           for (int x = 4; x < 32; ++x) mx4[x & 3] = fmaxf(mx4[x & 3], sc[x]);
           float mx = fmaxf(fmaxf(mx4[0], mx4[1]), fmaxf(mx4[2], mx4[3]));
-          mx = fmaxf(mx, __shfl_xor(mx, 32));
+          mx = fp::max_across_lane_halves(mx);
           // Lazy running maximum: the reference point m_run only moves when some row's maximum has
           // grown by more than kMaxSlack (log2 units); until then exp2(s - m_run) may reach
           // 2^kMaxSlack, harmless in bf16/f16 P and fp32 sums, and the accumulators need no rescale.

@@ -318,7 +318,7 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_f32_kernel(const Ar
         float mx = sc[0];
 #pragma unroll
         for (int x = 1; x < 16; ++x) mx = fmaxf(mx, sc[x]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        mx = fp::max_across_lane_halves(mx);
         // Lazy running maximum: the reference point m_run only moves when some row's maximum has grown by
         // more than kMaxSlack (log2 units); until then exp2(s - m_run) may reach 2^kMaxSlack, harmless in
         // fp32, and the accumulators need no rescale.
