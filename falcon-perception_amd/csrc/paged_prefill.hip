@@ -25,7 +25,7 @@
 // Rows of one tile may belong to several sequences: the tile is processed one
 // run of equal batch_idx at a time; rows of slot 0 are padding (out 0, lse -inf).
 #include "fp_common.h"
-#include "lds_dma.h"
+#include "prefill_common.h"
 
 #include <hip/hip_bf16.h>
 #include <hip/hip_fp16.h>

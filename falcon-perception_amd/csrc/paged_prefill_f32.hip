@@ -14,7 +14,7 @@
 //   O^T = V^T P^T : P^T is the B operand as it leaves the softmax; the A operand is read from the
 //                 row-major V tile one float per lane.
 #include "fp_common.h"
-#include "lds_dma.h"
+#include "prefill_common.h"
 
 #include <math.h>
 

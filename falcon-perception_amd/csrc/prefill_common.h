@@ -1,6 +1,7 @@
-// Loads from global memory straight into LDS (no staging registers), shared by the prefill kernels.
-#ifndef FP_LDS_DMA_H
-#define FP_LDS_DMA_H
+// Shared by the prefill kernels: loads from global memory straight into LDS (no staging registers)
+// and an exchange between the two halves of a wavefront.
+#ifndef FP_PREFILL_COMMON_H
+#define FP_PREFILL_COMMON_H
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
