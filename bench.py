@@ -205,6 +205,8 @@ PREFILL_WORKLOADS = {
     # whole sequences in one step (prefix 0): the image span rows are bidirectional
     "cfg3w": dict(seed=3, dtype="bf16", n_seq=8, Hq=16, Hc=8, D=128, P=128, prefix_lo=256, prefix_hi=4096, chunk=512,
                   whole=True),
+    # one request alone: a 512-token chunk over a 4096-token prefix (32 workgroups before the cut along the keys)
+    "cfg3one": dict(seed=3, dtype="bf16", n_seq=1, Hq=16, Hc=8, D=128, P=128, prefix_lo=4096, prefix_hi=4096, chunk=512),
     # cfg3 in the reference's default dtype (reference server/config.py:38)
     "cfg3f32": dict(seed=3, dtype="f32", n_seq=8, Hq=16, Hc=8, D=128, P=128, prefix_lo=256, prefix_hi=4096, chunk=512),
 }
@@ -250,7 +252,9 @@ class PrefillCase:
         from falcon_perception_amd import ops
 
         return ops.paged_prefill(self.q, self.pool_k, self.pool_v, self.cache.page_table, self.batch_idx,
-                                 self.row_limit, self.page_size)
+                                 self.row_limit, self.page_size,
+                                 workspace=self.cache.prefill_workspace(self.q.shape[2], self.q.shape[1], self.q.shape[3],
+                                                                        self.pool_k.shape[0], self.q.dtype))
 
     def run(self):
         self.append()
@@ -487,7 +491,9 @@ def prefill_rate(steps: int = 10, name: str = "cfg3") -> dict:
     what = {"cfg3": "cfg3: 8 sequences, paged prefix U[256,4096], 512-token chunk each, 16 q / 8 kv heads, D 128",
             "cfg3w": "cfg3w: the same 8 sequences prefilled whole (prefix + chunk rows in one step, prefix rows see "
                      "their whole image span), 16 q / 8 kv heads, D 128",
-            "cfg3f32": "cfg3 in fp32"}[name]
+            "cfg3f32": "cfg3 in fp32",
+            "cfg3one": "one sequence alone: paged prefix 4096, 512-token chunk, 16 q / 8 kv heads, D 128 "
+                       "(cut along the keys into 8 shares + merge pass)"}[name]
     res = {"workload": what, "query_rows": int(case.q.shape[2]), "paged_prefill_ms": ms, "tflops": tf,
            "chunk_append_ms": ms_a, "flops": case.flops()}
     if case.q.dtype == torch.float32:
@@ -631,6 +637,7 @@ def main() -> int:
         result["prefill_sized"] = append_gather_rates()
         result["chunked_prefill"] = prefill_rate()
         result["chunked_prefill_fp32"] = prefill_rate(name="cfg3f32")
+        result["chunked_prefill_one_sequence"] = prefill_rate(name="cfg3one")
         ms_model = model_depth_graph_ms(case, args.steps)  # last: it takes and returns 56 GiB
         if ms_model is not None:
             result["ms_all_layers_hip_graph"] = ms_model

@@ -45,6 +45,7 @@ constexpr float kLn2 = 0.6931471805599453f;
 
 typedef uint32_t v4u __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -69,6 +70,10 @@ struct PrefillArgs {
   int64_t n_slots;
   float qscale;  // scale * log2(e)
   int n_tiles;   // query tiles
+  // key split: grid z = n_key_splits workgroups share a query tile, each taking an equal share of every
+  // run's key tiles and leaving unnormalised partial results for the merge pass
+  float* ws_acc;  // [n_key_splits, Lq, Hq, D]
+  float* ws_ml;   // [n_key_splits, Lq, Hq, 2]: running maximum (log2 units), denominator
 };
 
 struct BF16 {
@@ -260,6 +265,13 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
         if (!active[mb]) continue;
+        if (gridDim.z > 1) {  // an empty share; the merge pass then writes out = 0, lse = -inf
+          const int64_t p = (static_cast<int64_t>(blockIdx.z) * a.Lq + row[mb]) * a.Hq + hq;
+#pragma unroll
+          for (int c = 0; c < D / 8; ++c) *reinterpret_cast<f32x4*>(a.ws_acc + p * D + half * (D / 2) + c * 4) = f32x4{0, 0, 0, 0};
+          if (half == 0) *reinterpret_cast<float2*>(a.ws_ml + p * 2) = float2{-INFINITY, 0.f};
+          continue;
+        }
         // a row is 2 * D bytes; each lane half clears D of them
         char* o = a.out + row[mb] * a.os_row + hq * a.os_h + half * D;
 #pragma unroll
@@ -289,7 +301,11 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) kv_max = max(kv_max, s_red[w]);
     kv_max = __builtin_amdgcn_readfirstlane(kv_max);
-    const int n_kv_tiles = (kv_max + kTileN - 1) / kTileN;
+    const int n_run_tiles = (kv_max + kTileN - 1) / kTileN;
+    // this workgroup's share of the run's key tiles: [kt_lo, n_kv_tiles)
+    const int kt_lo = static_cast<int>(static_cast<int64_t>(n_run_tiles) * blockIdx.z / gridDim.z);
+    const int n_kv_tiles = static_cast<int>(static_cast<int64_t>(n_run_tiles) * (blockIdx.z + 1) / gridDim.z);
+    const int n_my = n_kv_tiles - kt_lo;
 
     f32x16 o_acc[MB][DB];
     float m_run[MB], l_run[MB];
@@ -312,7 +328,7 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
     const int64_t* pt_row = a.page_table + static_cast<int64_t>(sq) * a.pt_row_stride;
     const int64_t pool_pages = a.n_slots / a.pd.page_size;
     const bool page_holds_tile = kPow2 && a.pd.page_size % kTileN == 0;
-    for (int t = tid; t < n_kv_tiles && t < kSlotTable; t += kThreads) {
+    for (int t = kt_lo + tid; t < n_kv_tiles && t - kt_lo < kSlotTable; t += kThreads) {
       int slot = -1;
       if (page_holds_tile && (t + 1) * kTileN <= kv_max) {
         const int key0 = t * kTileN;
@@ -322,12 +338,12 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
           if (pg >= 0 && pg < pool_pages) slot = static_cast<int>(pg) * a.pd.page_size + (key0 & (a.pd.page_size - 1));
         }
       }
-      s_tslot[t] = slot;
+      s_tslot[t - kt_lo] = slot;
     }
     __syncthreads();
     // first pool slot of tile kt, or -1: wavefront-uniform
     auto tile_slot = [&](int kt) {
-      return __builtin_amdgcn_readfirstlane((kt >= 0 && kt < n_kv_tiles && kt < kSlotTable) ? s_tslot[kt] : -1);
+      return __builtin_amdgcn_readfirstlane((kt >= kt_lo && kt < n_kv_tiles && kt - kt_lo < kSlotTable) ? s_tslot[kt - kt_lo] : -1);
     };
 
     auto key_block = [&](int kpos, int& blkid, int& off) {
@@ -389,9 +405,9 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
     // begins.  (A second barrier between the two parts of the interval kept the halves in step more
     // strictly and cost 2 %.)  K(i) lives in K buffer i % 2, V(i) in V buffer i % 2.
     {
-      const int ts0 = tile_slot(0);
+      const int ts0 = tile_slot(kt_lo);
 #pragma unroll
-      for (int piece = NI; piece < 2 * NI; ++piece) fetch_piece(piece, 0, ts0, s_k0);  // K(0)
+      for (int piece = NI; piece < 2 * NI; ++piece) fetch_piece(piece, kt_lo, ts0, s_k0);  // K of the first tile
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's rows have landed in LDS
 
@@ -415,13 +431,13 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
       const char* vprev = kBuf ? s_v0 : s_v1;  // V(i - 1)
       char* knext = kBuf ? s_k0 : s_k1;        // K(i + 1) goes here
       char* vcur = kBuf ? s_v1 : s_v0;         // V(i) goes here
-      const int key0 = i * kTileN;
-      const bool work_cur = key0 < wave_max;
+      const int key0 = (kt_lo + i) * kTileN;  // step i works on key tile kt_lo + i
+      const bool work_cur = i < n_my && key0 < wave_max;
       const bool work_prev = i > 0 && key0 - kTileN < wave_max;
 
       // the staging step this wavefront issues during the step: K of tile kt_k, V of tile kt_k - 1.
       // The table is read ahead of the barrier, whose wait hides the LDS latency.
-      const int kt_k = kSecond ? i + 2 : i + 1;
+      const int kt_k = kt_lo + (kSecond ? i + 2 : i + 1);
       const int ts_k = tile_slot(kt_k);
       const int ts_v = tile_slot(kt_k - 1);
       if (!kSecond) __builtin_amdgcn_s_waitcnt(0x0F70);  // staging step i - 1 of this wavefront has landed
@@ -570,24 +586,24 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
       }
     };
 
-    // steps 0 .. n_kv_tiles (the last one only has the O^T part of the last tile)
+    // steps 0 .. n_my (the last one only has the O^T part of the last tile)
     if (wave < kWaves / 2) {
-      for (int i = 0; i <= n_kv_tiles; i += 2) {
+      for (int i = 0; i <= n_my; i += 2) {
         step(IntC<0>{}, IntC<0>{}, i);
-        if (i + 1 <= n_kv_tiles) step(IntC<0>{}, IntC<1>{}, i + 1);
+        if (i + 1 <= n_my) step(IntC<0>{}, IntC<1>{}, i + 1);
       }
-      __builtin_amdgcn_s_barrier();  // the second half's last barrier, B(n_kv_tiles + 1)
+      __builtin_amdgcn_s_barrier();  // the second half's last barrier, B(n_my + 1)
     } else {
       __builtin_amdgcn_s_barrier();  // B(0): the first half starts M(0)
       {  // staging step 0: K(1), V(0)
-        const int ts1 = tile_slot(1), ts0 = tile_slot(0);
+        const int ts1 = tile_slot(kt_lo + 1), ts0 = tile_slot(kt_lo);
 #pragma unroll
         for (int piece = 0; piece < 2 * NI; ++piece)
-          fetch_piece(piece, piece < NI ? 0 : 1, piece < NI ? ts0 : ts1, piece < NI ? s_v0 : s_k1);
+          fetch_piece(piece, piece < NI ? kt_lo : kt_lo + 1, piece < NI ? ts0 : ts1, piece < NI ? s_v0 : s_k1);
       }
-      for (int i = 0; i <= n_kv_tiles; i += 2) {
+      for (int i = 0; i <= n_my; i += 2) {
         step(IntC<1>{}, IntC<0>{}, i);
-        if (i + 1 <= n_kv_tiles) step(IntC<1>{}, IntC<1>{}, i + 1);
+        if (i + 1 <= n_my) step(IntC<1>{}, IntC<1>{}, i + 1);
       }
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // no staging load is in flight when the LDS tiles are reused
@@ -598,6 +614,19 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
       const float l_tot = l_run[mb] + __shfl_xor(l_run[mb], 32);
       const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
       if (!active[mb]) continue;
+      if (gridDim.z > 1) {
+        // one of several key shares: the unnormalised state goes to the merge pass
+        const int64_t p = (static_cast<int64_t>(blockIdx.z) * a.Lq + row[mb]) * a.Hq + hq;
+        float* po = a.ws_acc + p * D;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int i4 = 0; i4 < 4; ++i4)
+            *reinterpret_cast<f32x4*>(po + db * 32 + i4 * 8 + half * 4) =
+                f32x4{o_acc[mb][db][i4 * 4], o_acc[mb][db][i4 * 4 + 1], o_acc[mb][db][i4 * 4 + 2], o_acc[mb][db][i4 * 4 + 3]};
+        if (half == 0) *reinterpret_cast<float2*>(a.ws_ml + p * 2) = float2{m_run[mb], l_tot};
+        continue;
+      }
       char* o = a.out + row[mb] * a.os_row + hq * a.os_h;
       const float lse_nat = l_tot > 0.f ? (m_run[mb] + log2f(l_tot)) * kLn2 : -INFINITY;
       // attention-sink gate of the caller's post-attention step (model.py:122-128): the output,
@@ -622,25 +651,115 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
   }
 }
 
+// ---- merge of the key shares ----
+// One wavefront per (query row, query head): combines the shares' unnormalised accumulators with
+// their running maxima and denominators, applies the sink gate, stores out and lse.
+constexpr int kMergeRows = 4;  // (row, head) pairs per workgroup
+
+template <typename E, int D>
+__global__ __launch_bounds__(kMergeRows * 64) void paged_prefill_merge_kernel(const PrefillArgs a, int n_shares) {
+  constexpr int EPL = D / 64;  // output elements per lane
+  const int lane = threadIdx.x & 63;
+  const int64_t item = static_cast<int64_t>(blockIdx.x) * kMergeRows + (threadIdx.x >> 6);
+  if (item >= static_cast<int64_t>(a.Lq) * a.Hq) return;
+  const int row = static_cast<int>(item / a.Hq), hq = static_cast<int>(item % a.Hq);
+  const int64_t share_stride = static_cast<int64_t>(a.Lq) * a.Hq;
+  constexpr int kBatch = 8;  // the launcher never makes more shares
+  float m_s[kBatch], l_s[kBatch], acc_s[kBatch][EPL];
+#pragma unroll
+  for (int s = 0; s < kBatch; ++s) {
+    const bool on = s < n_shares;
+    const int64_t p = s * share_stride + item;
+    m_s[s] = on ? a.ws_ml[p * 2] : -INFINITY;
+    l_s[s] = on ? a.ws_ml[p * 2 + 1] : 0.f;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) acc_s[s][e] = on ? a.ws_acc[p * D + lane * EPL + e] : 0.f;
+  }
+  float mn = -INFINITY;
+#pragma unroll
+  for (int s = 0; s < kBatch; ++s) mn = fmaxf(mn, m_s[s]);
+  const float ms = mn == -INFINITY ? 0.f : mn;
+  float den = 0.f, num[EPL];
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) num[e] = 0.f;
+#pragma unroll
+  for (int s = 0; s < kBatch; ++s) {
+    const float wgt = fast_exp2(m_s[s] - ms);  // 0 for a share that saw no key
+    den += l_s[s] * wgt;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) num[e] += acc_s[s][e] * wgt;
+  }
+  const float inv = den > 0.f ? 1.f / den : 0.f;
+  const float lse_nat = den > 0.f ? (mn + log2f(den)) * kLn2 : -INFINITY;
+  const bool gated = a.sinks != nullptr;
+  const float gate = gated ? 1.f / (1.f + __expf(a.sinks[hq] - lse_nat)) : 1.f;
+  auto fin = [&](float x) { return gated ? E::round(x * inv) * gate : x * inv; };
+  char* o = a.out + row * a.os_row + hq * a.os_h + lane * EPL * 2;
+  if (EPL == 2)
+    *reinterpret_cast<uint32_t*>(o) = E::pack2(fin(num[0]), fin(num[EPL - 1]));
+  else
+    *reinterpret_cast<short*>(o) = E::from_float(fin(num[0]));
+  if (lane == 0) a.lse[static_cast<int64_t>(hq) * a.Lq + row] = lse_nat;
+}
+
+// CUs of the current device (asked once per device; the answer never changes)
+int compute_units() {
+  static int cached[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
+constexpr int kMaxKeyShares = 8;
+
+// Key shares for a launch of `wgs` workgroups: a launch that would leave at least half of the CUs idle is
+// cut along the keys until every CU has a workgroup.  (With about one workgroup per CU already, a cut in
+// two costs more in partial results and their merge than the shorter critical path saves: 138 us
+// against 111 us at 8 sequences x 512 rows.)
+int key_shares_for(int64_t wgs) {
+  const int64_t n = compute_units() / (wgs > 0 ? wgs : 1);
+  return static_cast<int>(n < 1 ? 1 : n > kMaxKeyShares ? kMaxKeyShares : n);
+}
+
+int64_t share_bytes(int shares, int Lq, int Hq, int D) {
+  return shares <= 1 ? 0 : static_cast<int64_t>(shares) * Lq * Hq * (D + 2) * static_cast<int64_t>(sizeof(float));
+}
+
 template <typename E, int D, int G>
-void launch_group(const PrefillArgs& a0, hipStream_t st) {
+void launch_group(const PrefillArgs& a0, void* workspace, int64_t workspace_bytes, hipStream_t st) {
   PrefillArgs a = a0;
   constexpr int BM = (kWaves / G) * 32;
   a.n_tiles = (a.Lq + BM - 1) / BM;
-  dim3 grid(a.Hc, a.n_tiles);
+  int shares = workspace ? key_shares_for(static_cast<int64_t>(a.Hc) * a.n_tiles) : 1;
+  while (shares > 1 && share_bytes(shares, a.Lq, a.Hq, D) > workspace_bytes) --shares;  // what the workspace holds
+  if (shares > 1) {
+    a.ws_acc = static_cast<float*>(workspace);
+    a.ws_ml = a.ws_acc + static_cast<int64_t>(shares) * a.Lq * a.Hq * D;
+  }
+  dim3 grid(a.Hc, a.n_tiles, shares);
   if (a.pd.shift >= 0)
     hipLaunchKernelGGL((paged_prefill_kernel<E, D, G, true>), grid, dim3(kThreads), 0, st, a);
   else
     hipLaunchKernelGGL((paged_prefill_kernel<E, D, G, false>), grid, dim3(kThreads), 0, st, a);
+  if (shares > 1) {
+    const int64_t items = static_cast<int64_t>(a.Lq) * a.Hq;
+    hipLaunchKernelGGL((paged_prefill_merge_kernel<E, D>), dim3(static_cast<unsigned>((items + kMergeRows - 1) / kMergeRows)),
+                       dim3(kMergeRows * 64), 0, st, a, shares);
+  }
 }
 
 template <typename E, int D>
-int launch(const PrefillArgs& a, hipStream_t st) {
+int launch(const PrefillArgs& a, void* ws, int64_t ws_bytes, hipStream_t st) {
   switch (a.Hq / a.Hc) {
-    case 1: launch_group<E, D, 1>(a, st); return FP_OK;
-    case 2: launch_group<E, D, 2>(a, st); return FP_OK;
-    case 4: launch_group<E, D, 4>(a, st); return FP_OK;
-    case 8: launch_group<E, D, 8>(a, st); return FP_OK;
+    case 1: launch_group<E, D, 1>(a, ws, ws_bytes, st); return FP_OK;
+    case 2: launch_group<E, D, 2>(a, ws, ws_bytes, st); return FP_OK;
+    case 4: launch_group<E, D, 4>(a, ws, ws_bytes, st); return FP_OK;
+    case 8: launch_group<E, D, 8>(a, ws, ws_bytes, st); return FP_OK;
     default: return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill: Hq/Hc = %d (supported: 1, 2, 4, 8)", a.Hq / a.Hc);
   }
 }
@@ -653,7 +772,8 @@ extern "C" int fp_paged_prefill(const void* q, int64_t q_stride_row, int64_t q_s
                                 int64_t out_stride_row, int64_t out_stride_h, float* lse, const float* sinks,
                                 int32_t Lq, int32_t Hq,
                                 int32_t Hc, int32_t D, int32_t page_size, int32_t n_pages, int32_t max_batch,
-                                int64_t n_slots, float scale, int dtype, void* stream) {
+                                int64_t n_slots, float scale, int dtype, void* workspace, int64_t workspace_bytes,
+                                void* stream) {
   if (dtype != FP_DTYPE_BF16 && dtype != FP_DTYPE_F16 && dtype != FP_DTYPE_F32)
     return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill: unknown dtype %d", dtype);
   if (D != 64 && D != 128) return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill: head_dim %d (supported: 64, 128)", D);
@@ -686,13 +806,28 @@ extern "C" int fp_paged_prefill(const void* q, int64_t q_stride_row, int64_t q_s
                 static_cast<const char*>(pool_k), static_cast<const char*>(pool_v),
                 page_table, pt_row_stride, batch_idx, row_limit,
                 static_cast<char*>(out), out_stride_row * 2, out_stride_h * 2, lse, sinks,
-                Lq, Hq, Hc, fp::PageDiv(page_size), n_pages, max_batch, n_slots, scale * kLog2e, 0};
+                Lq, Hq, Hc, fp::PageDiv(page_size), n_pages, max_batch, n_slots, scale * kLog2e, 0, nullptr, nullptr};
+  if (workspace && (!fp::aligned(workspace, 16) || workspace_bytes < 0))
+    return fp::fail(FP_ERR_WORKSPACE, "fp_paged_prefill: the workspace must be 16-byte aligned");
   hipStream_t st = static_cast<hipStream_t>(stream);
   int rc;
   if (dtype == FP_DTYPE_BF16)
-    rc = D == 64 ? launch<BF16, 64>(a, st) : launch<BF16, 128>(a, st);
+    rc = D == 64 ? launch<BF16, 64>(a, workspace, workspace_bytes, st) : launch<BF16, 128>(a, workspace, workspace_bytes, st);
   else
-    rc = D == 64 ? launch<F16, 64>(a, st) : launch<F16, 128>(a, st);
+    rc = D == 64 ? launch<F16, 64>(a, workspace, workspace_bytes, st) : launch<F16, 128>(a, workspace, workspace_bytes, st);
   if (rc != FP_OK) return rc;
   return fp::check_launch("fp_paged_prefill");
+}
+
+extern "C" int64_t fp_paged_prefill_workspace_bytes(int32_t Lq, int32_t Hq, int32_t Hc, int32_t D, int dtype) {
+  if (Lq < 0 || Hq <= 0 || Hc <= 0 || Hq % Hc || (D != 64 && D != 128))
+    return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_prefill_workspace_bytes: bad dimension");
+  const int g = Hq / Hc;
+  if (g != 1 && g != 2 && g != 4 && g != 8)
+    return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill_workspace_bytes: Hq/Hc = %d (supported: 1, 2, 4, 8)", g);
+  if (dtype == FP_DTYPE_F32 || Lq == 0) return 0;  // the fp32 kernel does not split along the keys
+  if (dtype != FP_DTYPE_BF16 && dtype != FP_DTYPE_F16)
+    return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill_workspace_bytes: unknown dtype %d", dtype);
+  const int bm = (kWaves / g) * 32;
+  return share_bytes(key_shares_for(static_cast<int64_t>(Hc) * ((Lq + bm - 1) / bm)), Lq, Hq, D);
 }

@@ -254,10 +254,12 @@ def hybrid_row_limits(input_ids: Tensor, soi_id: int, eoi_id: int) -> Tensor:
 def paged_prefill(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor, batch_idx: Tensor,
                   row_limit: Tensor, page_size: int, *, scale: float | None = None,
                   out: Tensor | None = None, lse: Tensor | None = None,
-                  sinks: Tensor | None = None) -> tuple[Tensor, Tensor]:
+                  sinks: Tensor | None = None, workspace: Tensor | None | bool = None) -> tuple[Tensor, Tensor]:
     """Chunked-prefill attention over the paged cache.  q [1, Hq, Lq, D]; row r sees keys
     0..row_limit[r]-1 of sequence batch_idx[r]; returns out like q, lse [1, Hq, Lq].
-    `sinks` [Hq] float32 gates the output as in `paged_decode`."""
+    `sinks` [Hq] float32 gates the output as in `paged_decode`.  `workspace`: a uint8 tensor of
+    `prefill_workspace_bytes(...)` bytes lets a launch too small for the GPU be cut along the keys as
+    well; None allocates one when the shape calls for it, False runs without."""
     N.require_cuda(q, pool_k, pool_v, page_table, batch_idx, row_limit, out, lse)
     one, Hq, Lq, D = q.shape
     if one != 1:
@@ -280,11 +282,28 @@ def paged_prefill(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor,
         lse = torch.empty((1, Hq, Lq), dtype=torch.float32, device=q.device)
     if out.stride(3) != 1 or not lse.is_contiguous():
         raise RuntimeError("out rows must be dense and lse contiguous")
+    if workspace is None:
+        need = prefill_workspace_bytes(Lq, Hq, Hc, D, q.dtype)
+        workspace = torch.empty(need, dtype=torch.uint8, device=q.device) if need else False
+    ws_ptr, ws_bytes = None, 0
+    if workspace is not False:
+        N.require_cuda(workspace)
+        if workspace.dtype != torch.uint8 or not workspace.is_contiguous():
+            raise RuntimeError("workspace must be a contiguous uint8 tensor")
+        ws_ptr, ws_bytes = workspace.data_ptr(), workspace.numel()
     rc = N.lib().fp_paged_prefill(
         q.data_ptr(), q.stride(2), q.stride(1), pool_k.data_ptr(), pool_v.data_ptr(),
         page_table.data_ptr(), page_table.stride(0), batch_idx.data_ptr(),
         row_limit.data_ptr(), out.data_ptr(), out.stride(2), out.stride(1), lse.data_ptr(),
         _sinks_ptr(sinks, Hq, q.device), Lq, Hq, Hc, D, page_size, page_table.shape[1], page_table.shape[0], n_slots,
-        scale, N.dtype_code(q.dtype), N.stream_ptr(q.device))
+        scale, N.dtype_code(q.dtype), ws_ptr, ws_bytes, N.stream_ptr(q.device))
     N.check(rc, "fp_paged_prefill")
     return out, lse
+
+
+def prefill_workspace_bytes(Lq: int, Hq: int, Hc: int, D: int, dtype: torch.dtype) -> int:
+    """Bytes of workspace with which `paged_prefill` cuts a launch of this shape along the keys as finely as
+    it would like to on the current device (0: it would not cut it)."""
+    n = int(N.lib().fp_paged_prefill_workspace_bytes(Lq, Hq, Hc, D, N.dtype_code(dtype)))
+    N.check(n, "fp_paged_prefill_workspace_bytes")
+    return n

@@ -85,6 +85,7 @@ class PagedKVCache(KVCacheBase):
         self.last_decode_step: StepMeta | None = None
         self.last_prefill_step: StepMeta | None = None
         self._workspace: Tensor | None = None
+        self._prefill_workspace: Tensor | None = None
 
     # ------------------------------------------------------------------ append
     def insert_kv(self, layer_id: int, k: Tensor, v: Tensor, input_pos: Tensor | None = None,
@@ -317,3 +318,13 @@ class PagedKVCache(KVCacheBase):
         if self._workspace is None or self._workspace.numel() < need:
             self._workspace = torch.empty(need, dtype=torch.uint8, device=self.kv_cache.device)
         return self._workspace
+
+    def prefill_workspace(self, Lq: int, Hq: int, D: int, Hc: int, dtype: torch.dtype):
+        """Scratch with which the prefill kernel cuts a small launch along the keys as well, owned by the
+        cache and grown on demand (prefill steps are not captured in graphs); False when the shape needs none."""
+        need = ops.prefill_workspace_bytes(Lq, Hq, Hc, D, dtype)
+        if need == 0:
+            return False
+        if self._prefill_workspace is None or self._prefill_workspace.numel() < need:
+            self._prefill_workspace = torch.empty(need, dtype=torch.uint8, device=self.kv_cache.device)
+        return self._prefill_workspace

@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define FP_ABI_VERSION 2
+#define FP_ABI_VERSION 3
 
 /* element types of pool / q / k / v */
 #define FP_DTYPE_F32 0
@@ -313,7 +313,17 @@ int fp_hybrid_row_limits(const int64_t* input_ids, int32_t L,
  *              every such key must already be in the pages
  *   out        [Lq, Hq, D] view, strides (row, head); lse [Hq, Lq] float32
  *   sinks      NULL, or [Hq] float32 attention-sink logits, as in fp_paged_decode
+ *   workspace  NULL, or workspace_bytes bytes of device memory, 16-byte aligned (no need to clear it).
+ *              A launch with fewer workgroups than the GPU needs (few query rows, few heads) is then
+ *              also cut along the keys: up to 8 workgroups share a query tile, each takes an equal part
+ *              of the keys, and a merge pass combines them (two launches instead of one).  Without a
+ *              workspace, or with one that is too small, the cut is coarser or absent; results agree
+ *              within rounding.  fp32 never uses it.
  */
+/* Bytes of workspace with which fp_paged_prefill cuts a launch of this shape as finely as it would like
+ * to on the current device (0: it would not cut it at all); a negative FP_ERR_* for a bad argument. */
+int64_t fp_paged_prefill_workspace_bytes(int32_t Lq, int32_t Hq, int32_t Hc, int32_t D, int dtype);
+
 int fp_paged_prefill(const void* q, int64_t q_stride_row, int64_t q_stride_h,
                      const void* pool_k, const void* pool_v,
                      const int64_t* page_table, int64_t pt_row_stride,
@@ -323,6 +333,7 @@ int fp_paged_prefill(const void* q, int64_t q_stride_row, int64_t q_stride_h,
                      int32_t Lq, int32_t Hq, int32_t Hc, int32_t D,
                      int32_t page_size, int32_t n_pages, int32_t max_batch,
                      int64_t n_slots, float scale, int dtype,
+                     void* workspace, int64_t workspace_bytes,
                      void* stream);
 
 #ifdef __cplusplus
