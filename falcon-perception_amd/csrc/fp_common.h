@@ -59,6 +59,12 @@ int prefill_mfma_f32(const void* q, int64_t q_stride_row, int64_t q_stride_h, co
                      const int64_t* page_table, int64_t pt_row_stride, const int64_t* batch_idx,
                      const int32_t* row_limit, void* out, int64_t out_stride_row, int64_t out_stride_h, float* lse,
                      const float* sinks, int32_t Lq, int32_t Hq, int32_t Hc, int32_t D, int32_t page_size,
-                     int32_t n_pages, int32_t max_batch, int64_t n_slots, float scale, hipStream_t st);
+                     int32_t n_pages, int32_t max_batch, int64_t n_slots, float scale, void* workspace,
+                     int64_t workspace_bytes, hipStream_t st);
+
+// Key shares the prefill kernel of `dtype` cuts a launch of `wgs` workgroups into on the current device
+// (1 .. 8), and the workspace bytes `shares` of them need (paged_prefill.hip)
+int prefill_key_shares(int64_t wgs, int dtype);
+int64_t prefill_share_bytes(int shares, int Lq, int Hq, int D);
 
 }  // namespace fp

@@ -717,12 +717,16 @@ int compute_units() {
 
 constexpr int kMaxKeyShares = 8;
 
-// Key shares for a launch of `wgs` workgroups: a launch that would leave at least half of the CUs idle is
-// cut along the keys until every CU has a workgroup.  (With about one workgroup per CU already, a cut in
-// two costs more in partial results and their merge than the shorter critical path saves: 138 us
-// against 111 us at 8 sequences x 512 rows.)
-int key_shares_for(int64_t wgs) {
-  const int64_t n = compute_units() / (wgs > 0 ? wgs : 1);
+// Key shares for a launch of `wgs` workgroups.  bf16 / f16: a launch that would leave at least half of the
+// CUs idle is cut along the keys until every CU has a workgroup.  (With about one workgroup per CU
+// already, a cut in two costs more in partial results and their merge than the shorter critical path
+// saves: 138 us against 111 us at 8 sequences x 512 rows.)  fp32: the kernel takes about eight times as
+// long over the same partial results, so the cut pays until there are about four workgroups per CU to
+// even out sequences of different lengths and the last, partly filled round of workgroups (8 sequences
+// x 512 rows: 962 us uncut, 838 us in four shares; one sequence of 4608 rows: 1992 us and 1315 us).
+int key_shares_for(int64_t wgs, int dtype) {
+  if (wgs < 1) wgs = 1;
+  const int64_t n = dtype == FP_DTYPE_F32 ? (4 * compute_units() + wgs / 2) / wgs : compute_units() / wgs;
   return static_cast<int>(n < 1 ? 1 : n > kMaxKeyShares ? kMaxKeyShares : n);
 }
 
@@ -735,7 +739,7 @@ void launch_group(const PrefillArgs& a0, void* workspace, int64_t workspace_byte
   PrefillArgs a = a0;
   constexpr int BM = (kWaves / G) * 32;
   a.n_tiles = (a.Lq + BM - 1) / BM;
-  int shares = workspace ? key_shares_for(static_cast<int64_t>(a.Hc) * a.n_tiles) : 1;
+  int shares = workspace ? key_shares_for(static_cast<int64_t>(a.Hc) * a.n_tiles, FP_DTYPE_BF16) : 1;  // f16 alike
   while (shares > 1 && share_bytes(shares, a.Lq, a.Hq, D) > workspace_bytes) --shares;  // what the workspace holds
   if (shares > 1) {
     a.ws_acc = static_cast<float*>(workspace);
@@ -787,6 +791,8 @@ extern "C" int fp_paged_prefill(const void* q, int64_t q_stride_row, int64_t q_s
   if (Lq == 0) return FP_OK;
   if (!q || !pool_k || !pool_v || !page_table || !batch_idx || !row_limit || !out || !lse)
     return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_prefill: null pointer");
+  if (workspace && (!fp::aligned(workspace, 16) || workspace_bytes < 0))
+    return fp::fail(FP_ERR_WORKSPACE, "fp_paged_prefill: the workspace must be 16-byte aligned");
   if (dtype == FP_DTYPE_F32) {
     // fp32 has a kernel of its own on the fp32 matrix instruction
     if (!fp::aligned(q, 16) || !fp::aligned(pool_k, 16) || !fp::aligned(pool_v, 16) || !fp::aligned(out, 4) ||
@@ -794,7 +800,8 @@ extern "C" int fp_paged_prefill(const void* q, int64_t q_stride_row, int64_t q_s
       return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_prefill: q rows must be 16-byte aligned");
     const int rc32 = fp::prefill_mfma_f32(q, q_stride_row, q_stride_h, pool_k, pool_v, page_table, pt_row_stride, batch_idx,
                                           row_limit, out, out_stride_row, out_stride_h, lse, sinks, Lq, Hq, Hc, D, page_size,
-                                          n_pages, max_batch, n_slots, scale, static_cast<hipStream_t>(stream));
+                                          n_pages, max_batch, n_slots, scale, workspace, workspace_bytes,
+                                          static_cast<hipStream_t>(stream));
     if (rc32 != FP_OK) return rc32;
     return fp::check_launch("fp_paged_prefill");
   }
@@ -807,8 +814,6 @@ extern "C" int fp_paged_prefill(const void* q, int64_t q_stride_row, int64_t q_s
                 page_table, pt_row_stride, batch_idx, row_limit,
                 static_cast<char*>(out), out_stride_row * 2, out_stride_h * 2, lse, sinks,
                 Lq, Hq, Hc, fp::PageDiv(page_size), n_pages, max_batch, n_slots, scale * kLog2e, 0, nullptr, nullptr};
-  if (workspace && (!fp::aligned(workspace, 16) || workspace_bytes < 0))
-    return fp::fail(FP_ERR_WORKSPACE, "fp_paged_prefill: the workspace must be 16-byte aligned");
   hipStream_t st = static_cast<hipStream_t>(stream);
   int rc;
   if (dtype == FP_DTYPE_BF16)
@@ -825,9 +830,12 @@ extern "C" int64_t fp_paged_prefill_workspace_bytes(int32_t Lq, int32_t Hq, int3
   const int g = Hq / Hc;
   if (g != 1 && g != 2 && g != 4 && g != 8)
     return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill_workspace_bytes: Hq/Hc = %d (supported: 1, 2, 4, 8)", g);
-  if (dtype == FP_DTYPE_F32 || Lq == 0) return 0;  // the fp32 kernel does not split along the keys
-  if (dtype != FP_DTYPE_BF16 && dtype != FP_DTYPE_F16)
+  if (Lq == 0) return 0;
+  if (dtype != FP_DTYPE_BF16 && dtype != FP_DTYPE_F16 && dtype != FP_DTYPE_F32)
     return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill_workspace_bytes: unknown dtype %d", dtype);
   const int bm = (kWaves / g) * 32;
-  return share_bytes(key_shares_for(static_cast<int64_t>(Hc) * ((Lq + bm - 1) / bm)), Lq, Hq, D);
+  return share_bytes(key_shares_for(static_cast<int64_t>(Hc) * ((Lq + bm - 1) / bm), dtype), Lq, Hq, D);
 }
+
+int fp::prefill_key_shares(int64_t wgs, int dtype) { return key_shares_for(wgs, dtype); }
+int64_t fp::prefill_share_bytes(int shares, int Lq, int Hq, int D) { return share_bytes(shares, Lq, Hq, D); }

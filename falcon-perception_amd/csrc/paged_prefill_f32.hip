@@ -60,6 +60,9 @@ struct Args {
   int64_t n_slots;
   float qscale;  // scale * log2(e)
   int n_tiles;   // query tiles
+  // key shares (grid z): unnormalised partial results for the merge pass, as in the bf16 / f16 kernel
+  float* ws_acc;  // [shares, Lq, Hq, D]
+  float* ws_ml;   // [shares, Lq, Hq, 2]: running maximum (log2 units), denominator
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -182,7 +185,12 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_f32_kernel(const Ar
 
     if (sq == 0) {
       // padding rows: out = 0, lse = -inf; each lane half clears half of the row
-      if (active) {
+      if (active && gridDim.z > 1) {  // an empty share; the merge pass then writes out = 0, lse = -inf
+        const int64_t p = (static_cast<int64_t>(blockIdx.z) * a.Lq + row) * a.Hq + hq;
+#pragma unroll
+        for (int c = 0; c < D / 8; ++c) *reinterpret_cast<f32x4*>(a.ws_acc + p * D + half * (D / 2) + c * 4) = f32x4{0, 0, 0, 0};
+        if (half == 0) *reinterpret_cast<float2*>(a.ws_ml + p * 2) = float2{-INFINITY, 0.f};
+      } else if (active) {
         float* o = reinterpret_cast<float*>(a.out + row * a.os_row + hq * a.os_h) + half * (D / 2);
 #pragma unroll
         for (int c = 0; c < D / 2; ++c) o[c] = 0.f;
@@ -208,7 +216,10 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_f32_kernel(const Ar
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) kv_max = max(kv_max, s_red[w]);
     kv_max = __builtin_amdgcn_readfirstlane(kv_max);
-    const int n_kv_tiles = (kv_max + kTileN - 1) / kTileN;
+    const int n_run_tiles = (kv_max + kTileN - 1) / kTileN;
+    // this workgroup's share of the run's key tiles: [kt_lo, n_kv_tiles)
+    const int kt_lo = static_cast<int>(static_cast<int64_t>(n_run_tiles) * blockIdx.z / gridDim.z);
+    const int n_kv_tiles = static_cast<int>(static_cast<int64_t>(n_run_tiles) * (blockIdx.z + 1) / gridDim.z);
 
     f32x16 o_acc[DB];
 #pragma unroll
@@ -226,7 +237,7 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_f32_kernel(const Ar
     const int64_t* pt_row = a.page_table + static_cast<int64_t>(sq) * a.pt_row_stride;
     const int64_t pool_pages = a.n_slots / a.pd.page_size;
     const bool page_holds_tile = kPow2 && a.pd.page_size % kTileN == 0;
-    for (int t = tid; t < n_kv_tiles && t < kSlotTable; t += kThreads) {
+    for (int t = kt_lo + tid; t < n_kv_tiles && t - kt_lo < kSlotTable; t += kThreads) {
       int slot = -1;
       if (page_holds_tile && (t + 1) * kTileN <= kv_max) {
         const int key0 = t * kTileN;
@@ -236,12 +247,12 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_f32_kernel(const Ar
           if (pg >= 0 && pg < pool_pages) slot = static_cast<int>(pg) * a.pd.page_size + (key0 & (a.pd.page_size - 1));
         }
       }
-      s_tslot[t] = slot;
+      s_tslot[t - kt_lo] = slot;
     }
     __syncthreads();
     // first pool slot of tile kt, or -1: wavefront-uniform
     auto tile_slot = [&](int kt) {
-      return __builtin_amdgcn_readfirstlane((kt >= 0 && kt < n_kv_tiles && kt < kSlotTable) ? s_tslot[kt] : -1);
+      return __builtin_amdgcn_readfirstlane((kt >= kt_lo && kt < n_kv_tiles && kt - kt_lo < kSlotTable) ? s_tslot[kt - kt_lo] : -1);
     };
     auto key_block = [&](int kpos, int& blkid, int& off) {
       if (kPow2) {  // page size is a power of two: shift and mask, no branch on the page size
@@ -277,7 +288,7 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_f32_kernel(const Ar
       }
     };
 
-    stage(0, tile_slot(0), s_k0, s_v0);
+    stage(kt_lo, tile_slot(kt_lo), s_k0, s_v0);
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's rows have landed in LDS
     __syncthreads();
 
@@ -361,7 +372,7 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_f32_kernel(const Ar
       __syncthreads();
     };
 
-    for (int kt = 0; kt < n_kv_tiles; kt += 2) {
+    for (int kt = kt_lo; kt < n_kv_tiles; kt += 2) {
       tile_step(IntC<0>{}, kt);
       if (kt + 1 < n_kv_tiles) tile_step(IntC<1>{}, kt + 1);
     }
@@ -370,7 +381,18 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_f32_kernel(const Ar
     {
       const float l_tot = l_run + __shfl_xor(l_run, 32);
       const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-      if (active) {
+      if (active && gridDim.z > 1) {
+        // one of several key shares: the unnormalised state goes to the merge pass
+        const int64_t p = (static_cast<int64_t>(blockIdx.z) * a.Lq + row) * a.Hq + hq;
+        float* po = a.ws_acc + p * D;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int i4 = 0; i4 < 4; ++i4)
+            *reinterpret_cast<f32x4*>(po + db * 32 + i4 * 8 + half * 4) =
+                f32x4{o_acc[db][i4 * 4], o_acc[db][i4 * 4 + 1], o_acc[db][i4 * 4 + 2], o_acc[db][i4 * 4 + 3]};
+        if (half == 0) *reinterpret_cast<float2*>(a.ws_ml + p * 2) = float2{m_run, l_tot};
+      } else if (active) {
         float* o = reinterpret_cast<float*>(a.out + row * a.os_row + hq * a.os_h);
         const float lse_nat = l_tot > 0.f ? (m_run + log2f(l_tot)) * kLn2 : -INFINITY;
         // attention-sink gate of the caller's post-attention step (model.py:122-128)
@@ -391,25 +413,81 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_f32_kernel(const Ar
   }
 }
 
+// ---- merge of the key shares: one wavefront per (query row, query head) ----
+constexpr int kMergeRows = 4;  // (row, head) pairs per workgroup
+
+template <int D>
+__global__ __launch_bounds__(kMergeRows * 64) void paged_prefill_f32_merge_kernel(const Args a, int n_shares) {
+  constexpr int EPL = D / 64;  // output elements per lane
+  const int lane = threadIdx.x & 63;
+  const int64_t item = static_cast<int64_t>(blockIdx.x) * kMergeRows + (threadIdx.x >> 6);
+  if (item >= static_cast<int64_t>(a.Lq) * a.Hq) return;
+  const int row = static_cast<int>(item / a.Hq), hq = static_cast<int>(item % a.Hq);
+  const int64_t share_stride = static_cast<int64_t>(a.Lq) * a.Hq;
+  constexpr int kBatch = 8;  // the launcher never makes more shares
+  float m_s[kBatch], l_s[kBatch], acc_s[kBatch][EPL];
+#pragma unroll
+  for (int s = 0; s < kBatch; ++s) {
+    const bool on = s < n_shares;
+    const int64_t p = s * share_stride + item;
+    m_s[s] = on ? a.ws_ml[p * 2] : -INFINITY;
+    l_s[s] = on ? a.ws_ml[p * 2 + 1] : 0.f;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) acc_s[s][e] = on ? a.ws_acc[p * D + lane * EPL + e] : 0.f;
+  }
+  float mn = -INFINITY;
+#pragma unroll
+  for (int s = 0; s < kBatch; ++s) mn = fmaxf(mn, m_s[s]);
+  const float ms = mn == -INFINITY ? 0.f : mn;
+  float den = 0.f, num[EPL];
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) num[e] = 0.f;
+#pragma unroll
+  for (int s = 0; s < kBatch; ++s) {
+    const float wgt = fast_exp2(m_s[s] - ms);  // 0 for a share that saw no key
+    den += l_s[s] * wgt;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) num[e] += acc_s[s][e] * wgt;
+  }
+  const float lse_nat = den > 0.f ? (mn + log2f(den)) * kLn2 : -INFINITY;
+  const float gate = a.sinks != nullptr ? 1.f / (1.f + __expf(a.sinks[hq] - lse_nat)) : 1.f;
+  const float f = (den > 0.f ? 1.f / den : 0.f) * gate;
+  float* o = reinterpret_cast<float*>(a.out + row * a.os_row + hq * a.os_h) + lane * EPL;
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) o[e] = num[e] * f;
+  if (lane == 0) a.lse[static_cast<int64_t>(hq) * a.Lq + row] = lse_nat;
+}
+
 template <int D, int G>
-void launch_group(const Args& a0, hipStream_t st) {
+void launch_group(const Args& a0, void* workspace, int64_t workspace_bytes, hipStream_t st) {
   Args a = a0;
   constexpr int BM = (kWaves / G) * 32;
   a.n_tiles = (a.Lq + BM - 1) / BM;
-  dim3 grid(a.Hc, a.n_tiles);
+  int shares = workspace ? fp::prefill_key_shares(static_cast<int64_t>(a.Hc) * a.n_tiles, FP_DTYPE_F32) : 1;
+  while (shares > 1 && fp::prefill_share_bytes(shares, a.Lq, a.Hq, D) > workspace_bytes) --shares;
+  if (shares > 1) {
+    a.ws_acc = static_cast<float*>(workspace);
+    a.ws_ml = a.ws_acc + static_cast<int64_t>(shares) * a.Lq * a.Hq * D;
+  }
+  dim3 grid(a.Hc, a.n_tiles, shares);
   if (a.pd.shift >= 0)
     hipLaunchKernelGGL((paged_prefill_f32_kernel<D, G, true>), grid, dim3(kThreads), 0, st, a);
   else
     hipLaunchKernelGGL((paged_prefill_f32_kernel<D, G, false>), grid, dim3(kThreads), 0, st, a);
+  if (shares > 1) {
+    const int64_t items = static_cast<int64_t>(a.Lq) * a.Hq;
+    hipLaunchKernelGGL((paged_prefill_f32_merge_kernel<D>), dim3(static_cast<unsigned>((items + kMergeRows - 1) / kMergeRows)),
+                       dim3(kMergeRows * 64), 0, st, a, shares);
+  }
 }
 
 template <int D>
-int launch(const Args& a, hipStream_t st) {
+int launch(const Args& a, void* ws, int64_t ws_bytes, hipStream_t st) {
   switch (a.Hq / a.Hc) {
-    case 1: launch_group<D, 1>(a, st); return FP_OK;
-    case 2: launch_group<D, 2>(a, st); return FP_OK;
-    case 4: launch_group<D, 4>(a, st); return FP_OK;
-    case 8: launch_group<D, 8>(a, st); return FP_OK;
+    case 1: launch_group<D, 1>(a, ws, ws_bytes, st); return FP_OK;
+    case 2: launch_group<D, 2>(a, ws, ws_bytes, st); return FP_OK;
+    case 4: launch_group<D, 4>(a, ws, ws_bytes, st); return FP_OK;
+    case 8: launch_group<D, 8>(a, ws, ws_bytes, st); return FP_OK;
     default: return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill: Hq/Hc = %d (supported: 1, 2, 4, 8)", a.Hq / a.Hc);
   }
 }
@@ -422,14 +500,15 @@ int prefill_mfma_f32(const void* q, int64_t q_stride_row, int64_t q_stride_h, co
                      const int64_t* page_table, int64_t pt_row_stride, const int64_t* batch_idx,
                      const int32_t* row_limit, void* out, int64_t out_stride_row, int64_t out_stride_h, float* lse,
                      const float* sinks, int32_t Lq, int32_t Hq, int32_t Hc, int32_t D, int32_t page_size,
-                     int32_t n_pages, int32_t max_batch, int64_t n_slots, float scale, hipStream_t st) {
+                     int32_t n_pages, int32_t max_batch, int64_t n_slots, float scale, void* workspace,
+                     int64_t workspace_bytes, hipStream_t st) {
   if ((static_cast<int64_t>(Lq) + 31) / 32 > 65535) return fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill: too many query rows");
   Args a{static_cast<const char*>(q), q_stride_row * 4, q_stride_h * 4,
          static_cast<const char*>(pool_k), static_cast<const char*>(pool_v),
          page_table, pt_row_stride, batch_idx, row_limit,
          static_cast<char*>(out), out_stride_row * 4, out_stride_h * 4, lse, sinks,
-         Lq, Hq, Hc, PageDiv(page_size), n_pages, max_batch, n_slots, scale * kLog2e, 0};
-  return D == 64 ? launch<64>(a, st) : launch<128>(a, st);
+         Lq, Hq, Hc, PageDiv(page_size), n_pages, max_batch, n_slots, scale * kLog2e, 0, nullptr, nullptr};
+  return D == 64 ? launch<64>(a, workspace, workspace_bytes, st) : launch<128>(a, workspace, workspace_bytes, st);
 }
 
 }  // namespace fp

@@ -318,7 +318,7 @@ int fp_hybrid_row_limits(const int64_t* input_ids, int32_t L,
  *              also cut along the keys: up to 8 workgroups share a query tile, each takes an equal part
  *              of the keys, and a merge pass combines them (two launches instead of one).  Without a
  *              workspace, or with one that is too small, the cut is coarser or absent; results agree
- *              within rounding.  fp32 never uses it.
+ *              within rounding.
  */
 /* Bytes of workspace with which fp_paged_prefill cuts a launch of this shape as finely as it would like
  * to on the current device (0: it would not cut it at all); a negative FP_ERR_* for a bad argument. */
