@@ -503,6 +503,23 @@ def prefill_rate(steps: int = 10, name: str = "cfg3") -> dict:
     return res
 
 
+def small_batch_decode(steps: int = 200) -> dict:
+    """The decode step (append + split-K pass + merge pass) of a few long sequences, replayed from a HIP
+    graph: the regime of one or a few requests, where the split length and the merge pass set the time."""
+    out = {}
+    for B, L in ((1, 8192), (1, 32768), (4, 8192), (16, 8192)):
+        name = f"small_B{B}_L{L}"
+        DECODE_WORKLOADS[name] = dict(seed=7, dtype="bf16", B=B, Hq=16, Hc=8, D=128, P=128,
+                                      n_pages=B * (L // 128 + 2) + 8, prefix=L - 64, lo=0, hi=63)
+        case = make_decode_case(name)
+        ms = graph_ms(case.run_fused, steps)
+        out[f"batch {B}, context ~{L}"] = {"split_tokens": case.split_tokens, "ms_per_step_hip_graph": ms,
+                                          "gbps": case.bytes_decode() / (ms * 1e-3) / 1e9}
+        del DECODE_WORKLOADS[name], case
+        torch.cuda.empty_cache()
+    return out
+
+
 def cpu_baseline(case: DecodeCase, budget_s: float = 20.0) -> dict:
     """The reference's op sequence for one decode layer-step, ported to torch-CPU, timed on the
     host cores on a batch subset sized to roughly `budget_s` seconds."""
@@ -638,6 +655,7 @@ def main() -> int:
         result["chunked_prefill"] = prefill_rate()
         result["chunked_prefill_fp32"] = prefill_rate(name="cfg3f32")
         result["chunked_prefill_one_sequence"] = prefill_rate(name="cfg3one")
+        result["decode_small_batch"] = small_batch_decode()
         ms_model = model_depth_graph_ms(case, args.steps)  # last: it takes and returns 56 GiB
         if ms_model is not None:
             result["ms_all_layers_hip_graph"] = ms_model

@@ -486,6 +486,60 @@ __global__ __launch_bounds__(kThreads) void paged_decode_kernel(const DecodeArgs
 }
 
 // ---- cross-split merge ------------------------------------------------------
+// Folds the splits first, first + stride, ... (kBatch consecutive splits each time, below ns) of partial
+// row p0 into the running state (m_run, den, num) of this lane; scores are in log2 units.
+template <int D, int kBatch>
+__device__ __forceinline__ void merge_batches(const DecodeArgs& a, int64_t p0, int first, int stride, int ns, float& m_run,
+                                              float& den, float (&num)[(D + 63) / 64]) {
+  constexpr int DPL = (D + 63) / 64;
+  for (int base = first; base < ns; base += stride) {
+    float m_s[kBatch], l_s[kBatch], acc_s[kBatch][DPL];
+#pragma unroll
+    for (int s = 0; s < kBatch; ++s) {
+      const bool on = base + s < ns;
+      const int64_t p = p0 + (on ? base + s : 0);
+      m_s[s] = on ? a.ws_ml[p * 2] : -INFINITY;
+      l_s[s] = on ? a.ws_ml[p * 2 + 1] : 0.f;
+#pragma unroll
+      for (int j = 0; j < DPL; ++j) {
+        const int d = (threadIdx.x & 63) + j * 64;
+        acc_s[s][j] = (on && d < D) ? a.ws_acc[p * D + d] : 0.f;
+      }
+    }
+    float mn = m_run;
+#pragma unroll
+    for (int s = 0; s < kBatch; ++s) mn = fmaxf(mn, m_s[s]);
+    const float ms = safe_max(mn);
+    const float keep = fast_exp2(m_run - ms);  // 0 while the state is empty
+    den *= keep;
+#pragma unroll
+    for (int j = 0; j < DPL; ++j) num[j] *= keep;
+#pragma unroll
+    for (int s = 0; s < kBatch; ++s) {
+      const float wgt = fast_exp2(m_s[s] - ms);
+      den += l_s[s] * wgt;
+#pragma unroll
+      for (int j = 0; j < DPL; ++j) num[j] += acc_s[s][j] * wgt;
+    }
+    m_run = mn;
+  }
+}
+
+// Normalises, gates and stores one merged row (lane = output elements lane, lane + 64, ...).
+template <typename E, int D>
+__device__ __forceinline__ void finish_merge(const DecodeArgs& a, int b, int hq, bool any, float mn, float den,
+                                             const float (&num)[(D + 63) / 64]) {
+  const float lse_nat = any ? (mn + log2f(den)) * kLn2 : -INFINITY;
+#pragma unroll
+  for (int j = 0; j < (D + 63) / 64; ++j) {
+    const int d = (threadIdx.x & 63) + j * 64;
+    if (d >= D) continue;
+    const float o = any ? num[j] / den : 0.f;
+    E::store(a.out + b * a.os_b + hq * a.os_h + d * sizeof(typename E::type), sink_gate<E>(o, lse_nat, a.sinks, hq));
+  }
+  if ((threadIdx.x & 63) == 0) a.lse[static_cast<int64_t>(b) * a.Hq + hq] = lse_nat;
+}
+
 template <typename E, int D>
 __global__ __launch_bounds__(64) void paged_decode_merge_kernel(const DecodeArgs a) {
   const int hq = blockIdx.x;
@@ -552,20 +606,66 @@ __global__ __launch_bounds__(64) void paged_decode_merge_kernel(const DecodeArgs
     return;
   }
 
-  float mn = -INFINITY;
-  for (int s = 0; s < ns; ++s) mn = fmaxf(mn, a.ws_ml[(p0 + s) * 2]);
-  const float ms = safe_max(mn);
-  float den = 0.f;
-  for (int s = 0; s < ns; ++s) den += a.ws_ml[(p0 + s) * 2 + 1] * fast_exp2(a.ws_ml[(p0 + s) * 2] - ms);
+  // More splits than one batch (launches over long contexts): the same lane keeps a running (maximum,
+  // denominator, numerator) over batches of kBatch splits, every load of a batch requested at once.  The
+  // wide variant of this kernel spreads the batches over several wavefronts.
+  float m_run = -INFINITY, den = 0.f, num[DPL];
+#pragma unroll
+  for (int j = 0; j < DPL; ++j) num[j] = 0.f;
+  merge_batches<D, kBatch>(a, p0, 0, kBatch, ns, m_run, den, num);
+  finish_merge<E, D>(a, b, hq, ns > 0, m_run, den, num);
+}
 
-  const float lse_nat = ns > 0 ? (mn + log2f(den)) * kLn2 : -INFINITY;
-  for (int d = threadIdx.x; d < D; d += 64) {
-    float num = 0.f;
-    for (int s = 0; s < ns; ++s) num += a.ws_acc[(p0 + s) * D + d] * fast_exp2(a.ws_ml[(p0 + s) * 2] - ms);
-    const float o = ns > 0 ? num / den : 0.f;
-    E::store(a.out + b * a.os_b + hq * a.os_h + d * sizeof(typename E::type), sink_gate<E>(o, lse_nat, a.sinks, hq));
+// Cross-split merge for launches with many splits per sequence: kMergeWideWaves wavefronts per
+// (sequence, query head) take the batches of splits round-robin and combine their states through LDS.
+constexpr int kMergeWideWaves = 8;
+constexpr int kMergeWideSplits = 16;  // launches with more splits than this use it
+
+template <typename E, int D>
+__global__ __launch_bounds__(kMergeWideWaves * 64) void paged_decode_merge_wide_kernel(const DecodeArgs a) {
+  constexpr int kBatch = 8;
+  constexpr int DPL = (D + 63) / 64;
+  const int hq = blockIdx.x;
+  const int b = blockIdx.y;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int64_t p0 = (static_cast<int64_t>(b) * a.Hq + hq) * a.n_splits;
+  __shared__ float s_m[kMergeWideWaves], s_den[kMergeWideWaves], s_num[kMergeWideWaves][DPL * 64];
+
+  int64_t L = fp::load_index(a.input_pos, b, a.pos_i64) + 1;
+  const int64_t trow = a.batch_idx[b];
+  if (trow < 0 || trow >= a.max_batch) L = 0;
+  if (L > a.max_context) L = a.max_context;
+  const int part = split_part(static_cast<int>(L), a.split_tokens);
+  const int ns = L <= 0 ? 0 : static_cast<int>((L + part - 1) / part);
+
+  float m_run = -INFINITY, den = 0.f, num[DPL];
+#pragma unroll
+  for (int j = 0; j < DPL; ++j) num[j] = 0.f;
+  merge_batches<D, kBatch>(a, p0, wave * kBatch, kMergeWideWaves * kBatch, ns, m_run, den, num);
+  if (lane == 0) {
+    s_m[wave] = m_run;
+    s_den[wave] = den;
   }
-  if (threadIdx.x == 0) a.lse[static_cast<int64_t>(b) * a.Hq + hq] = lse_nat;
+#pragma unroll
+  for (int j = 0; j < DPL; ++j) s_num[wave][j * 64 + lane] = num[j];
+  __syncthreads();
+  if (wave != 0) return;
+  float mn = -INFINITY;
+#pragma unroll
+  for (int w = 0; w < kMergeWideWaves; ++w) mn = fmaxf(mn, s_m[w]);
+  const float ms = safe_max(mn);
+  den = 0.f;
+#pragma unroll
+  for (int j = 0; j < DPL; ++j) num[j] = 0.f;
+#pragma unroll
+  for (int w = 0; w < kMergeWideWaves; ++w) {
+    const float wgt = fast_exp2(s_m[w] - ms);  // 0 for a wavefront that had no split
+    den += s_den[w] * wgt;
+#pragma unroll
+    for (int j = 0; j < DPL; ++j) num[j] += s_num[w][j * 64 + lane] * wgt;
+  }
+  finish_merge<E, D>(a, b, hq, ns > 0, mn, den, num);
 }
 
 constexpr int kPhasePartial = 1;
@@ -591,8 +691,12 @@ void launch_decode(const DecodeArgs& a, int B, int phases, hipStream_t st) {
       else
         hipLaunchKernelGGL((paged_decode_kernel<E, D, G, false, false, kPerHeadK>), grid, dim3(kThreads), 0, st, a);
     }
-    if (phases & kPhaseMerge)
-      hipLaunchKernelGGL((paged_decode_merge_kernel<E, D>), dim3(a.Hq, B), dim3(64), 0, st, a);
+    if (phases & kPhaseMerge) {
+      if (a.n_splits > kMergeWideSplits)
+        hipLaunchKernelGGL((paged_decode_merge_wide_kernel<E, D>), dim3(a.Hq, B), dim3(kMergeWideWaves * 64), 0, st, a);
+      else
+        hipLaunchKernelGGL((paged_decode_merge_kernel<E, D>), dim3(a.Hq, B), dim3(64), 0, st, a);
+    }
   }
 }
 
@@ -623,11 +727,16 @@ int dispatch_dim(const DecodeArgs& a, int B, int D, int phases, int kv_rep, hipS
   }
 }
 
-// Largest split (fewest partials to merge, least per-workgroup overhead) that still yields about
-// 2048 workgroups when every sequence is at max_context: 8 per CU to fill 256 CUs three deep.
+// Largest split (fewest partials to merge, least per-workgroup overhead) that still yields enough
+// workgroups when every sequence is at max_context.  Enough is about 2048 (8 per CU) for a batch whose
+// sequences alone give every CU two workgroups: their lengths differ, and small pieces even that out.
+// A small batch wants larger pieces: from 512 workgroups (4 * B * Hc in between) the pass no longer gets
+// faster, and every further split is one more partial result to merge.
 int default_split_tokens(int B, int Hc, int max_context, int page_size) {
+  int64_t target = 4 * static_cast<int64_t>(B) * Hc;
+  target = target < 512 ? 512 : target > 2048 ? 2048 : target;
   int split = 2048;
-  while (split > 128 && static_cast<int64_t>(B) * Hc * ((max_context + split - 1) / split) < 2048) split >>= 1;
+  while (split > 128 && static_cast<int64_t>(B) * Hc * ((max_context + split - 1) / split) < target) split >>= 1;
   while (split / page_size + 2 > kMaxSplitPages) split >>= 1;
   return split < 64 ? 64 : split;
 }

@@ -258,20 +258,21 @@ def test_fused_append_decode_equals_append_then_decode(dtype, ctx):
     np.testing.assert_allclose(f64(outs[1][1]), f64(outs[0][1]), atol=1e-4, rtol=1e-4)
 
 
-@pytest.mark.parametrize("split_tokens,n_splits", [(64, 21), (192, 7), (128, 11)])
-def test_merge_pass_with_few_and_with_many_splits(split_tokens, n_splits):
-    """The merge pass requests every partial at once when the launch has up to 8 splits and walks
-    them in a loop beyond: both forms, sequences that fill all, some or one of the splits, and one
-    without any key."""
-    dtype = torch.bfloat16
-    st = PagedState(21, n_pages=64, page_size=32, max_batch=8, Hc=2, D=128, dtype=dtype)
-    for L in (1300, 65, 500, 1):
+@pytest.mark.parametrize("dtype,D", [(torch.bfloat16, 128), (torch.float32, 64)], ids=str)
+@pytest.mark.parametrize("longest,split_tokens,n_splits", [(1300, 192, 7), (1300, 128, 11), (1300, 64, 21), (6000, 64, 94)])
+def test_merge_pass_with_few_and_with_many_splits(longest, split_tokens, n_splits, dtype, D):
+    """The merge pass has three forms: every partial requested at once (up to 8 splits), one wavefront
+    walking batches of 8 (up to 16), and eight wavefronts sharing the batches (beyond; with 94 splits
+    some of them take two batches and some one).  Each with sequences that fill all, some or one of the
+    splits, and one without any key."""
+    st = PagedState(21, n_pages=256, page_size=32, max_batch=8, Hc=2, D=D, dtype=dtype)
+    for L in (longest, 65, 500, 1):
         st.add_sequence(L)
     st.prefill_random()
-    q = randn(st.gen, (4, 4, 1, 128), dtype)
-    pos = torch.tensor([1299, 64, 499, -1], dtype=torch.int32)
-    assert -(-1300 // split_tokens) == n_splits
-    out, lse = run_decode(st, q, pos, split_tokens=split_tokens, max_context=1300)
+    q = randn(st.gen, (4, 4, 1, D), dtype)
+    pos = torch.tensor([longest - 1, 64, 499, -1], dtype=torch.int32)
+    assert -(-longest // split_tokens) == n_splits
+    out, lse = run_decode(st, q, pos, split_tokens=split_tokens, max_context=longest)
     eo, el = oracle_decode(st, q[:3], pos[:3])
     assert_close(out[:3], lse[:3], eo, el, dtype)
     assert not out[3].any() and torch.isneginf(lse[3]).all()
