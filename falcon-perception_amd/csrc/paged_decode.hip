@@ -263,8 +263,15 @@ __device__ __forceinline__ void fold_rows(const v4u (&kreg)[GK][U], const v4u (&
 // K rows and ONE V row (the first copy), i.e. (G + 1) / 2G of the bytes an expanded read costs.
 constexpr int decode_loads_in_flight(int G, bool per_head_k) { return per_head_k && G >= 4 ? 4 : 8; }
 
+// Four workgroups per CU instead of three (at most 128 registers) where the kernel fits without spilling:
+// one query head per cache head, and two in fp32 (the 16-bit kernels keep twice the elements per lane).
+template <typename E, int D, int G, bool kPerHeadK>
+constexpr int decode_waves_per_simd() {
+  return (!kPerHeadK && (G == 1 || (G == 2 && sizeof(typename E::type) == 4))) ? 4 : 1;
+}
+
 template <typename E, int D, int G, bool kDirect, bool kAligned, bool kPerHeadK = false>
-__global__ __launch_bounds__(kThreads) void paged_decode_kernel(const DecodeArgs a) {
+__global__ __launch_bounds__(kThreads, (decode_waves_per_simd<E, D, G, kPerHeadK>())) void paged_decode_kernel(const DecodeArgs a) {
   constexpr int EPL = E::kEpl;          // elements per lane
   constexpr int TPR = D / EPL;          // lanes per row
   constexpr int RPW = 64 / TPR;         // rows per wavefront load
@@ -280,9 +287,14 @@ __global__ __launch_bounds__(kThreads) void paged_decode_kernel(const DecodeArgs
   // Workgroups are dealt to the 8 XCDs round-robin by linear id.  Heads run fastest:
   // every head of a sequence has the same amount of work, so each XCD gets an equal
   // share of the non-empty workgroups whatever the context lengths are.
+  // The workgroup dispatcher deals consecutive workgroups of an XCD to its four shader engines in turn
+  // and starts them in order, so with grid y = sequence every split of a sequence would land on the
+  // same engine and an engine's load would be the lengths of "its" sequences (12 % apart at 64
+  // sequences of 1 k to 4 k tokens).  Rotating the sequences by the split index spreads each sequence
+  // over the engines.
   const int hc = blockIdx.x;
-  const int b = blockIdx.y;
   const int split = blockIdx.z;
+  const int b = static_cast<int>((blockIdx.y + blockIdx.z) % gridDim.y);
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
