@@ -23,6 +23,9 @@ inline int elem_bytes(int dtype) {
   }
 }
 
+// CUs of the current device (asked once per device; the answer never changes)
+int compute_units();
+
 inline bool aligned(const void* p, int n) { return (reinterpret_cast<uintptr_t>(p) % n) == 0; }
 
 // log2 of x if x is a power of two, else -1

@@ -29,3 +29,15 @@ int check_launch(const char* what) {
 extern "C" int fp_abi_version(void) { return FP_ABI_VERSION; }
 
 extern "C" const char* fp_last_error(void) { return fp::error_buffer(); }
+
+int fp::compute_units() {
+  static int cached[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}

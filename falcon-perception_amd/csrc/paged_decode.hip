@@ -60,6 +60,8 @@ struct DecodeArgs {
   const char* k_new;
   const char* v_new;
   int64_t kn_b, kn_h, vn_b, vn_h;  // bytes
+  int B;         // sequences of the launch
+  int n_chunks;  // even cut (kFlat): workgroups per cache head
 };
 
 // ---- element access: 16 bytes of a row -----------------------------------
@@ -270,7 +272,59 @@ constexpr int decode_waves_per_simd() {
   return (!kPerHeadK && (G == 1 || (G == 2 && sizeof(typename E::type) == 4))) ? 4 : 1;
 }
 
-template <typename E, int D, int G, bool kDirect, bool kAligned, bool kPerHeadK = false>
+// Even cut of a launch (kFlat): the contexts of the launch, each rounded up to 64 tokens, are laid end
+// to end and cut into n_chunks pieces of equal length.  Sequence b starts at flat_start[b]; chunk c covers
+// [c * len, (c + 1) * len); a chunk that spans several sequences works through them one after another.
+constexpr int kFlatMaxB = 1024;
+
+// Start of every sequence on the flat axis -> s_start[0 .. B] (s_start[B] = total), by one wavefront.
+__device__ __forceinline__ void flat_starts(const DecodeArgs& a, int* s_start) {
+  if (threadIdx.x < 64) {
+    const int lane = threadIdx.x;
+    const int per = (a.B + 63) / 64;  // consecutive sequences per lane
+    int sum = 0;
+    for (int i = 0; i < per; ++i) {
+      const int b = lane * per + i;
+      int Lr = 0;
+      if (b < a.B) {
+        int64_t L = fp::load_index(a.input_pos, b, a.pos_i64) + 1;
+        const int64_t trow = a.batch_idx[b];
+        if (trow < 0 || trow >= a.max_batch || L < 0) L = 0;
+        if (L > a.max_context) L = a.max_context;
+        Lr = (static_cast<int>(L) + 63) & ~63;
+      }
+      sum += Lr;
+    }
+    int incl = sum;  // inclusive scan over the lanes
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const int up = __shfl_up(incl, off);
+      if (lane >= off) incl += up;
+    }
+    int run = incl - sum;
+    for (int i = 0; i < per; ++i) {
+      const int b = lane * per + i;
+      if (b > a.B) break;
+      s_start[b] = run;
+      if (b < a.B) {
+        int64_t L = fp::load_index(a.input_pos, b, a.pos_i64) + 1;
+        const int64_t trow = a.batch_idx[b];
+        if (trow < 0 || trow >= a.max_batch || L < 0) L = 0;
+        if (L > a.max_context) L = a.max_context;
+        run += (static_cast<int>(L) + 63) & ~63;
+      }
+    }
+    if (lane == 63 && a.B == 64 * per) s_start[a.B] = incl;
+  }
+}
+
+// tokens per chunk of the even cut
+__device__ __forceinline__ int flat_chunk_len(int total, int n_chunks) {
+  const int len = (total + n_chunks - 1) / n_chunks;
+  return len < 64 ? 64 : (len + 63) & ~63;
+}
+
+template <typename E, int D, int G, bool kDirect, bool kAligned, bool kPerHeadK = false, bool kFlat = false>
 __global__ __launch_bounds__(kThreads, (decode_waves_per_simd<E, D, G, kPerHeadK>())) void paged_decode_kernel(const DecodeArgs a) {
   constexpr int EPL = E::kEpl;          // elements per lane
   constexpr int TPR = D / EPL;          // lanes per row
@@ -293,14 +347,16 @@ __global__ __launch_bounds__(kThreads, (decode_waves_per_simd<E, D, G, kPerHeadK
   // sequences of 1 k to 4 k tokens).  Rotating the sequences by the split index spreads each sequence
   // over the engines.
   const int hc = blockIdx.x;
-  const int split = blockIdx.z;
-  const int b = static_cast<int>((blockIdx.y + blockIdx.z) % gridDim.y);
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
   const int grp = lane / TPR;  // row of this lane inside a wavefront load
   const int col = lane % TPR;  // 16-byte chunk of the row
 
+  // Tokens [t0, t0 + part) of sequence b; a partial result goes to row hq * part_mul + part_add of the
+  // workspace.
+  auto piece = [&](const int b, const int t0, const int part, const bool first, const int64_t part_mul,
+                   const int64_t part_add) {
   int64_t L = fp::load_index(a.input_pos, b, a.pos_i64) + 1;
   const int64_t trow = a.batch_idx[b];
   if (trow < 0 || trow >= a.max_batch) L = 0;
@@ -308,13 +364,8 @@ __global__ __launch_bounds__(kThreads, (decode_waves_per_simd<E, D, G, kPerHeadK
   auto lse_at = [&](int hq) -> float& {
     return a.lse[static_cast<int64_t>(b) * a.Hq + hq];
   };
-  // A context of L tokens is cut into ceil(L / split_tokens) parts of equal size (a multiple of
-  // 64 tokens), so the workgroups of one sequence carry the same load instead of leaving a short
-  // tail split.
-  const int part = split_part(static_cast<int>(L), a.split_tokens);
-  const int t0 = split * part;
   if (t0 >= L) {
-    if (kDirect && split == 0) {
+    if (kDirect && first) {
       // no visible key at all: out = 0, lse = -inf
       for (int i = tid; i < G * D; i += kThreads) {
         const int g = i / D, d = i - g * D;
@@ -487,12 +538,59 @@ __global__ __launch_bounds__(kThreads, (decode_waves_per_simd<E, D, G, kPerHeadK
       E::store(a.out + b * a.os_b + hq * a.os_h + d * sizeof(typename E::type), sink_gate<E>(num / den, lse_nat, a.sinks, hq));
       if (d == 0) lse_at(hq) = lse_nat;
     } else {
-      const int64_t p = (static_cast<int64_t>(b) * a.Hq + hq) * a.n_splits + split;
+      const int64_t p = hq * part_mul + part_add;
       a.ws_acc[p * D + d] = num;
       if (d == 0) {
         a.ws_ml[p * 2] = mn;
         a.ws_ml[p * 2 + 1] = den;
       }
+    }
+  }
+  };  // piece
+
+  if constexpr (!kFlat) {
+    // grid (Hc, B, splits).  A context of L tokens is cut into ceil(L / split_tokens) parts of equal
+    // size (a multiple of 64 tokens), so the workgroups of one sequence carry the same load instead of
+    // leaving a short tail split.
+    // The workgroup dispatcher deals consecutive workgroups of an XCD to its four shader engines in turn
+    // and starts them in order, so with grid y = sequence every split of a sequence would land on the
+    // same engine and an engine's load would be the lengths of "its" sequences (12 % apart at 64
+    // sequences of 1 k to 4 k tokens).  Rotating the sequences by the split index spreads each sequence
+    // over the engines.
+    const int split = blockIdx.z;
+    const int b = static_cast<int>((blockIdx.y + blockIdx.z) % gridDim.y);
+    int64_t L = fp::load_index(a.input_pos, b, a.pos_i64) + 1;
+    if (L > a.max_context) L = a.max_context;
+    const int part = split_part(static_cast<int>(L < 0 ? 0 : L), a.split_tokens);
+    piece(b, split * part, part, split == 0, a.n_splits, static_cast<int64_t>(b) * a.Hq * a.n_splits + split);
+  } else {
+    // grid (Hc, n_chunks): every workgroup streams the same number of rows, whatever the lengths are
+    __shared__ int s_start[kFlatMaxB + 1];
+    flat_starts(a, s_start);
+    __syncthreads();
+    const int total = s_start[a.B];
+    const int len = flat_chunk_len(total, a.n_chunks);
+    const int c = blockIdx.y;
+    const int64_t lo = static_cast<int64_t>(c) * len;
+    const int64_t hi = lo + len < total ? lo + len : total;
+    if (lo >= total) return;
+    // first sequence that ends after lo
+    int b = 0;
+    {
+      int left = 0, right = a.B - 1;
+      while (left < right) {
+        const int mid = (left + right) >> 1;
+        if (s_start[mid + 1] > lo) right = mid; else left = mid + 1;
+      }
+      b = left;
+    }
+    for (; b < a.B && s_start[b] < hi; ++b) {
+      const int begin = s_start[b], end = s_start[b + 1];
+      if (end == begin) continue;  // a sequence without keys has no piece; the merge pass writes its zeros
+      const int t0 = lo > begin ? static_cast<int>(lo - begin) : 0;
+      const int t1 = static_cast<int>((hi < end ? hi : end) - begin);
+      piece(b, t0, t1 - t0, false, 1, static_cast<int64_t>(c + b) * a.Hq);
+      __syncthreads();  // the LDS of the piece is free again
     }
   }
 }
@@ -502,14 +600,14 @@ __global__ __launch_bounds__(kThreads, (decode_waves_per_simd<E, D, G, kPerHeadK
 // row p0 into the running state (m_run, den, num) of this lane; scores are in log2 units.
 template <int D, int kBatch>
 __device__ __forceinline__ void merge_batches(const DecodeArgs& a, int64_t p0, int first, int stride, int ns, float& m_run,
-                                              float& den, float (&num)[(D + 63) / 64]) {
+                                              float& den, float (&num)[(D + 63) / 64], int64_t row_stride = 1) {
   constexpr int DPL = (D + 63) / 64;
   for (int base = first; base < ns; base += stride) {
     float m_s[kBatch], l_s[kBatch], acc_s[kBatch][DPL];
 #pragma unroll
     for (int s = 0; s < kBatch; ++s) {
       const bool on = base + s < ns;
-      const int64_t p = p0 + (on ? base + s : 0);
+      const int64_t p = p0 + (on ? base + s : 0) * row_stride;
       m_s[s] = on ? a.ws_ml[p * 2] : -INFINITY;
       l_s[s] = on ? a.ws_ml[p * 2 + 1] : 0.f;
 #pragma unroll
@@ -628,6 +726,41 @@ __global__ __launch_bounds__(64) void paged_decode_merge_kernel(const DecodeArgs
   finish_merge<E, D>(a, b, hq, ns > 0, m_run, den, num);
 }
 
+// Cross-split merge after the even cut: sequence b has one partial result per chunk it touches, in
+// workspace rows (chunk + b) * Hq + hq.
+template <typename E, int D>
+__global__ __launch_bounds__(64) void paged_decode_merge_flat_kernel(const DecodeArgs a) {
+  constexpr int DPL = (D + 63) / 64;
+  const int hq = blockIdx.x;
+  const int b = blockIdx.y;
+  const int lane = threadIdx.x;
+  int before = 0, total = 0, mine = 0;  // rounded lengths: of the sequences before b, of all, of b
+  for (int i = lane; i < a.B; i += 64) {
+    int64_t L = fp::load_index(a.input_pos, i, a.pos_i64) + 1;
+    const int64_t trow = a.batch_idx[i];
+    if (trow < 0 || trow >= a.max_batch || L < 0) L = 0;
+    if (L > a.max_context) L = a.max_context;
+    const int Lr = (static_cast<int>(L) + 63) & ~63;
+    total += Lr;
+    if (i < b) before += Lr;
+    if (i == b) mine = Lr;
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    total += __shfl_xor(total, off);
+    before += __shfl_xor(before, off);
+    mine += __shfl_xor(mine, off);
+  }
+  const int len = flat_chunk_len(total, a.n_chunks);
+  const int c_first = before / len;
+  const int ns = mine > 0 ? (before + mine - 1) / len - c_first + 1 : 0;
+  float m_run = -INFINITY, den = 0.f, num[DPL];
+#pragma unroll
+  for (int j = 0; j < DPL; ++j) num[j] = 0.f;
+  merge_batches<D, 8>(a, static_cast<int64_t>(c_first + b) * a.Hq + hq, 0, 8, ns, m_run, den, num, a.Hq);
+  finish_merge<E, D>(a, b, hq, ns > 0, m_run, den, num);
+}
+
 // Cross-split merge for launches with many splits per sequence: kMergeWideWaves wavefronts per
 // (sequence, query head) take the batches of splits round-robin and combine their states through LDS.
 constexpr int kMergeWideWaves = 8;
@@ -683,6 +816,23 @@ __global__ __launch_bounds__(kMergeWideWaves * 64) void paged_decode_merge_wide_
 constexpr int kPhasePartial = 1;
 constexpr int kPhaseMerge = 2;
 
+// Workgroups of the even-cut kernel the current device holds at once (asked once per kernel and device).
+template <typename E, int D, int G, bool kAligned, bool kPerHeadK>
+int resident_workgroups() {
+  const auto kernel = paged_decode_kernel<E, D, G, false, kAligned, kPerHeadK, true>;
+  static int cached[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  if (cached[dev] == 0) {
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kThreads, 0) != hipSuccess || per_cu <= 0)
+      cached[dev] = -1;
+    else
+      cached[dev] = per_cu * fp::compute_units();
+  }
+  return cached[dev] > 0 ? cached[dev] : 0;
+}
+
 template <typename E, int D, int G, bool kPerHeadK = false>
 void launch_decode(const DecodeArgs& a, int B, int phases, hipStream_t st) {
   dim3 grid(a.Hc, B, a.n_splits);  // a.Hc = workgroups per sequence and split: cache heads, or groups of G heads
@@ -697,14 +847,45 @@ void launch_decode(const DecodeArgs& a, int B, int phases, hipStream_t st) {
     else
       hipLaunchKernelGGL((paged_decode_kernel<E, D, G, true, false, kPerHeadK>), grid, dim3(kThreads), 0, st, a);
   } else {
+    // A 16-bit launch with more workgroups than the GPU holds at once is cut evenly instead: two chunks
+    // per CU, all of the same length, all resident from the start, so that every CU streams the same
+    // number of rows (split by split, the CUs end up with loads 25 % apart at 64 sequences of 1 k to
+    // 4 k tokens, and workgroups queue behind busy shader engines).  Measured at 64 sequences of 16 q /
+    // 8 kv heads, bf16, % of 8 TB/s for the step with 1 / 2 / 3 / 4 chunks per CU and split by split:
+    // D 128: 75.5 / 75.4 / 73.8 / 73.1 and 73.0; D 64: 67.2 / 68.3 / 68.1 / 63.7 and 67.1; 32 q heads:
+    // 63.9 / 70.6 / 64.2 / 67.9 and 67.2; 16-token pages: 70.0 / 74.4 / 73.9 / 68.9 and 72.6.  fp32 is
+    // faster split by split (D 128: 77.5 against 73.8 / 70.4 / 69.6 / 69.2) and stays so.  The even cut
+    // needs the lengths of at most kFlatMaxB sequences in LDS, a workspace row per (chunk + sequence),
+    // and chunks within the page-id table.
+    int n_chunks = 0;
+    {
+      const int resident = aligned ? resident_workgroups<E, D, G, true, kPerHeadK>()
+                                   : resident_workgroups<E, D, G, false, kPerHeadK>();
+      const int64_t wgs = static_cast<int64_t>(a.Hc) * B * a.n_splits;
+      const int chunks = 2 * fp::compute_units() / a.Hc;
+      if (sizeof(typename E::type) == 2 && chunks >= 1 && wgs > resident && B <= kFlatMaxB && chunks + B <= static_cast<int64_t>(B) * a.n_splits &&
+          (static_cast<int64_t>(B) * a.max_context / chunks + 128) / a.pd.page_size + 2 <= kMaxSplitPages)
+        n_chunks = chunks;
+    }
+    DecodeArgs af = a;
+    af.B = B;
+    af.n_chunks = n_chunks;
     if (phases & kPhasePartial) {
-      if (aligned)
+      if (n_chunks > 0) {
+        if (aligned)
+          hipLaunchKernelGGL((paged_decode_kernel<E, D, G, false, true, kPerHeadK, true>), dim3(a.Hc, n_chunks), dim3(kThreads), 0, st, af);
+        else
+          hipLaunchKernelGGL((paged_decode_kernel<E, D, G, false, false, kPerHeadK, true>), dim3(a.Hc, n_chunks), dim3(kThreads), 0, st, af);
+      } else if (aligned) {
         hipLaunchKernelGGL((paged_decode_kernel<E, D, G, false, true, kPerHeadK>), grid, dim3(kThreads), 0, st, a);
-      else
+      } else {
         hipLaunchKernelGGL((paged_decode_kernel<E, D, G, false, false, kPerHeadK>), grid, dim3(kThreads), 0, st, a);
+      }
     }
     if (phases & kPhaseMerge) {
-      if (a.n_splits > kMergeWideSplits)
+      if (n_chunks > 0)
+        hipLaunchKernelGGL((paged_decode_merge_flat_kernel<E, D>), dim3(a.Hq, B), dim3(64), 0, st, af);
+      else if (a.n_splits > kMergeWideSplits)
         hipLaunchKernelGGL((paged_decode_merge_wide_kernel<E, D>), dim3(a.Hq, B), dim3(kMergeWideWaves * 64), 0, st, a);
       else
         hipLaunchKernelGGL((paged_decode_merge_kernel<E, D>), dim3(a.Hq, B), dim3(64), 0, st, a);
@@ -834,7 +1015,7 @@ int decode_entry(int phases, const NewRows* fresh, const void* q, int64_t q_stri
                static_cast<char*>(out), out_stride_b * eb, out_stride_h * eb, lse, sinks,
                nullptr, nullptr, Hq, wg_heads, fp::PageDiv(page_size), n_pages, max_batch, n_slots,
                max_context, split_tokens, ns, scale * kLog2e,  // scores are kept in log2 units
-               nullptr, nullptr, 0, 0, 0, 0};
+               nullptr, nullptr, 0, 0, 0, 0, B, 0};
   if (fresh) {
     if (!fresh->k || !fresh->v) return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode_append: null k_new / v_new");
     if (!fp::aligned(fresh->k, 16) || !fp::aligned(fresh->v, 16) || (fresh->k_stride_b * eb) % 16 ||

@@ -702,19 +702,6 @@ __global__ __launch_bounds__(kMergeRows * 64) void paged_prefill_merge_kernel(co
   if (lane == 0) a.lse[static_cast<int64_t>(hq) * a.Lq + row] = lse_nat;
 }
 
-// CUs of the current device (asked once per device; the answer never changes)
-int compute_units() {
-  static int cached[64] = {};
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (cached[dev] == 0) {
-    int n = 0;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    cached[dev] = n;
-  }
-  return cached[dev];
-}
-
 constexpr int kMaxKeyShares = 8;
 
 // Key shares for a launch of `wgs` workgroups.  bf16 / f16: a launch that would leave at least half of the
@@ -726,7 +713,7 @@ constexpr int kMaxKeyShares = 8;
 // x 512 rows: 962 us uncut, 838 us in four shares; one sequence of 4608 rows: 1992 us and 1315 us).
 int key_shares_for(int64_t wgs, int dtype) {
   if (wgs < 1) wgs = 1;
-  const int64_t n = dtype == FP_DTYPE_F32 ? (4 * compute_units() + wgs / 2) / wgs : compute_units() / wgs;
+  const int64_t n = dtype == FP_DTYPE_F32 ? (4 * fp::compute_units() + wgs / 2) / wgs : fp::compute_units() / wgs;
   return static_cast<int>(n < 1 ? 1 : n > kMaxKeyShares ? kMaxKeyShares : n);
 }
 

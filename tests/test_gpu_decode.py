@@ -276,3 +276,58 @@ def test_merge_pass_with_few_and_with_many_splits(longest, split_tokens, n_split
     eo, el = oracle_decode(st, q[:3], pos[:3])
     assert_close(out[:3], lse[:3], eo, el, dtype)
     assert not out[3].any() and torch.isneginf(lse[3]).all()
+
+
+@pytest.mark.parametrize("dtype,D,P,G", [(torch.bfloat16, 128, 64, 2), (torch.float32, 64, 16, 1), (torch.float16, 128, 48, 4)],
+                         ids=str)
+def test_a_launch_larger_than_the_gpu_is_cut_evenly(dtype, D, P, G):
+    """8 cache heads x 72 sequences x 8 splits = 4608 workgroups, more than the GPU holds at once: the
+    contexts are laid end to end and cut into equal chunks instead (about 190 tokens here), so chunks span
+    several short sequences and long sequences span several chunks.  Sequences of 1 token, of exactly one
+    chunk-rounding unit, one without any key and one at the maximum; fused append; the two passes called
+    separately; the same launch replayed from a graph."""
+    B, Hc, split, ctx = 72, 8, 64, 512
+    st = PagedState(33, n_pages=B * (-(-ctx // P)) + 8, page_size=P, max_batch=B + 2, Hc=Hc, D=D, dtype=dtype)
+    lens = torch.randint(0, ctx - 1, (B,), generator=st.gen).tolist()  # tokens cached before the step
+    lens[0], lens[1], lens[2], lens[3], lens[40] = ctx - 1, 0, 63, 64, 0
+    for L in lens:
+        st.add_sequence(L + 1)
+    st.lens = lens
+    st.prefill_random()
+    q = randn(st.gen, (B, Hc * G, 1, D), dtype)
+    k_new = randn(st.gen, (B, Hc, 1, D), dtype).to(DEV)
+    v_new = randn(st.gen, (B, Hc, 1, D), dtype).to(DEV)
+    pos = torch.tensor(lens, dtype=torch.int32)  # the new token's position
+    kw = dict(split_tokens=split, max_context=ctx)
+    out, lse = run_decode(st, q, pos, k_new=k_new, v_new=v_new, **kw)
+    eo, el = oracle_decode(st, q, pos)  # the pool now holds the new rows
+    assert_close(out, lse, eo, el, dtype)
+    # without the append (the rows are in the pool), one sequence masked out, passes called separately
+    pos2 = pos.clone()
+    pos2[5] = -1
+    need = ops.decode_workspace_bytes(B, Hc * G, D, ctx, split)
+    ws = torch.full((need,), 0xA5, dtype=torch.uint8, device=DEV)
+    run_decode(st, q, pos2, workspace=ws, phase="partial", **kw)
+    out2, lse2 = run_decode(st, q, pos2, workspace=ws, phase="merge", **kw)
+    keep = [i for i in range(B) if i != 5]  # their chunks lie elsewhere now: same values within rounding
+    assert_close(out2[keep], lse2[keep], eo[keep], el[keep], dtype)
+    assert not out2[5].any() and torch.isneginf(lse2[5]).all()
+    # from a graph, replayed
+    qd, bidx, posd = q.to(DEV), torch.tensor(st.slots, dtype=torch.int64, device=DEV), pos.to(DEV)
+    pk, pv = st.pool_planes()
+    out_g, lse_g = torch.empty_like(out), torch.empty_like(lse)
+    call = lambda: ops.paged_decode(qd, pk, pv, st.cache.page_table, bidx, posd, st.P, ctx, split_tokens=split,
+                                    workspace=ws, out=out_g, lse=lse_g, k_new=k_new, v_new=v_new)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call()
+    torch.cuda.current_stream().wait_stream(side)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        call()
+    for _ in range(3):
+        out_g.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, out) and torch.equal(lse_g, lse)
