@@ -49,7 +49,7 @@ DTYPES = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
 
 # HBM bytes per launch of paged_decode_kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # (profiles/), scaled by the same counters on a plain copy of known size; None = not measured
-TRAFFIC_BYTES = {"cfg2": 671.9e6}  # profiles/paged_decode_cfg2_hbm_traffic.md
+TRAFFIC_BYTES = {"cfg2": 671.4e6}  # profiles/paged_decode_cfg2_hbm_traffic.md
 
 
 @dataclass

@@ -184,11 +184,14 @@ int fp_paged_decode(const void* q, int64_t q_stride_b, int64_t q_stride_h,
 
 /*
  * The two passes of fp_paged_decode as separate calls, same arguments: the partial pass
- * leaves, per (sequence, query head, split), the unnormalised accumulator, running
- * maximum and denominator in the workspace ([B, Hq, n_splits, D] floats followed by
- * [B, Hq, n_splits, 2] floats, log2 units); the merge pass combines them into out and
- * lse.  For callers that time or overlap the passes, or that combine partials of one
- * sequence held on several devices with the same merge.  No counterpart in the
+ * leaves, per (sequence, query head, piece of the context), the unnormalised accumulator,
+ * running maximum and denominator in the workspace (log2 units); the merge pass combines
+ * them into out and lse.  The pieces are the splits of split_tokens tokens
+ * ([B, Hq, n_splits, D] floats followed by [B, Hq, n_splits, 2] floats), except that a 16-bit
+ * launch of more workgroups than the GPU holds at once is cut into equal chunks of the
+ * contexts laid end to end (rows (chunk + sequence) * Hq + head of [rows, D] and [rows, 2]
+ * floats): the layout is a matter between the two passes.  For callers that time or
+ * overlap the passes.  No counterpart in the
  * reference, whose Triton decode kernel keeps both passes internal
  * (torch/_inductor/kernel/flex/flex_decoding.py:229).  When one split covers
  * max_context the partial pass writes out and lse itself and the merge pass does nothing.
