@@ -92,3 +92,30 @@ def test_kv_rep_is_validated():
         ops.paged_decode(q, pk, pv, st.cache.page_table, bidx, pos, 16, 64, kv_rep=3)
     with pytest.raises(RuntimeError, match="one head per query head"):
         ops.paged_decode(q, pk[:2], pv[:2], st.cache.page_table, bidx, pos, 16, 64, kv_rep=2)
+
+
+def test_shared_v_and_sink_gate_through_the_even_cut():
+    """A launch of more workgroups than the GPU holds at once (80 sequences x 8 groups x 8 splits) is cut
+    into equal chunks of the flattened contexts; the shared-V read and the sink gate go through that path
+    and its merge pass too."""
+    dtype, P, rep, B = torch.bfloat16, 64, 2, 80
+    gen = torch.Generator().manual_seed(53)
+    lens = torch.randint(1, 500, (B,), generator=gen).tolist()
+    lens[0], lens[1] = 0, 511
+    st, Hq = expanded_state(53, rep, dtype, P, lens, Hkv=8)
+    q = randn(st.gen, (B, Hq, 1, 128), dtype).to(DEV)
+    pos = torch.tensor(lens, dtype=torch.int32, device=DEV) - 1
+    bidx = torch.tensor(st.slots, dtype=torch.int64, device=DEV)
+    sinks = torch.linspace(-2.0, 2.0, Hq, device=DEV)
+    pk, pv = st.pool_planes()
+    args = (q, pk, pv, st.cache.page_table, bidx, pos, P, 512)
+    out, lse = ops.paged_decode(*args, split_tokens=64, kv_rep=rep)
+    gated, lse_g = ops.paged_decode(*args, split_tokens=64, kv_rep=rep, sinks=sinks)
+    atol, rtol = TOL[dtype]
+    eo, el = O.decode_attention(f64(q), f64(pk), f64(pv), st.mirror.page_table, st.slots, pos.cpu().numpy(), P)
+    np.testing.assert_allclose(f64(out), eo, atol=atol, rtol=rtol)
+    np.testing.assert_allclose(f64(lse), el, atol=max(atol * 0.1, 2e-5), rtol=rtol)
+    assert torch.equal(lse_g, lse)
+    gate = 1.0 / (1.0 + np.exp(f64(sinks)[None, :, None] - f64(lse)))
+    np.testing.assert_allclose(f64(gated), f64(out) * gate[..., None], atol=atol, rtol=rtol)
+    assert not f64(out)[0].any() and np.isneginf(f64(lse)[0]).all()  # the sequence without keys
