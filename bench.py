@@ -447,6 +447,31 @@ def append_gather_rates(steps: int = 20, T: int = 32768, H: int = 16, D: int = 1
         ms_t = event_ms(do_part, steps)
         sweep[str(t)] = {"ms": ms_t, "gbps": (2 * t * (2 * H * D * e) + 8 * t) / (ms_t * 1e-3) / 1e9}
 
+    # The same append with nothing left in the last-level cache from the launch before: six pools and six
+    # sets of source rows taken in turn (3 GiB touched between two uses of the same addresses, against
+    # 256 MB of cache).  The figures above rewrite one pool from one set of rows.
+    rings = [(pk, pv, k_rows, v_rows, cache.page_table)]
+    for i in range(5):
+        c2 = PagedKVCache(T // P + 16, P, 4, H, D, 1, dtype, device=dev)
+        c2.free_pages = (torch.randperm(c2.n_pages - 1, generator=g) + 1).tolist()
+        b2 = c2.allocate()
+        assert b2 == b
+        c2.reserve(b2, torch.tensor([b2], device=dev), T)
+        k2 = torch.randn((T, H, D), device=dev, dtype=dtype)
+        v2 = torch.randn((T, H, D), device=dev, dtype=dtype)
+        rings.append((c2.kv_cache[0, 0, 0], c2.kv_cache[0, 1, 0], k2.unsqueeze(2), v2.unsqueeze(2), c2.page_table))
+    turn = [0]
+
+    def do_append_cold():
+        rk, rv, sk, sv, table = rings[turn[0] % len(rings)]
+        turn[0] += 1
+        ops.kv_append(rk, rv, sk, sv, table, flat_b, flat_p, P, clamp_negative=False)
+
+    for _ in range(len(rings)):
+        do_append_cold()
+    ms_cold = event_ms(do_append_cold, 3 * len(rings))
+    del rings
+
     # QK norm + rotary embedding + insert in one launch (reference model.py:110-119 + the append):
     # the qkv projection output of the same step, 16 query heads / 8 kv heads, expanded to the 16 cached heads
     Hkv = H // 2
@@ -474,6 +499,8 @@ def append_gather_rates(steps: int = 20, T: int = 32768, H: int = 16, D: int = 1
             "qkv_norm_rope_append_frac_of_peak": bytes_r / (ms_r * 1e-3) / 1e9 / HBM_PEAK_GBPS,
             "kv_append_ms": ms_a, "kv_append_gbps": bytes_a / (ms_a * 1e-3) / 1e9,
             "kv_append_frac_of_peak": bytes_a / (ms_a * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "kv_append_cold_ms": ms_cold, "kv_append_cold_gbps": bytes_a / (ms_cold * 1e-3) / 1e9,
+            "kv_append_cold_frac_of_peak": bytes_a / (ms_cold * 1e-3) / 1e9 / HBM_PEAK_GBPS,
             "kv_append_by_tokens": sweep,
             "kv_gather_ms": ms_g, "kv_gather_gbps": bytes_g / (ms_g * 1e-3) / 1e9,
             "kv_gather_frac_of_peak": bytes_g / (ms_g * 1e-3) / 1e9 / HBM_PEAK_GBPS}
