@@ -447,10 +447,11 @@ def append_gather_rates(steps: int = 20, T: int = 32768, H: int = 16, D: int = 1
         ms_t = event_ms(do_part, steps)
         sweep[str(t)] = {"ms": ms_t, "gbps": (2 * t * (2 * H * D * e) + 8 * t) / (ms_t * 1e-3) / 1e9}
 
-    # The same append with nothing left in the last-level cache from the launch before: six pools and six
-    # sets of source rows taken in turn (3 GiB touched between two uses of the same addresses, against
-    # 256 MB of cache).  The figures above rewrite one pool from one set of rows.
-    rings = [(pk, pv, k_rows, v_rows, cache.page_table)]
+    # The same append and gather with nothing left in the last-level cache from the launch before: six
+    # pools, six sets of source rows and six outputs taken in turn (3 GiB / 1.5 GiB touched between two
+    # uses of the same addresses, against 256 MB of cache).  The figures above rewrite one pool from one
+    # set of rows and gather one pool into one output.
+    rings = [(pk, pv, k_rows, v_rows, cache.page_table, out)]
     for i in range(5):
         c2 = PagedKVCache(T // P + 16, P, 4, H, D, 1, dtype, device=dev)
         c2.free_pages = (torch.randperm(c2.n_pages - 1, generator=g) + 1).tolist()
@@ -459,17 +460,24 @@ def append_gather_rates(steps: int = 20, T: int = 32768, H: int = 16, D: int = 1
         c2.reserve(b2, torch.tensor([b2], device=dev), T)
         k2 = torch.randn((T, H, D), device=dev, dtype=dtype)
         v2 = torch.randn((T, H, D), device=dev, dtype=dtype)
-        rings.append((c2.kv_cache[0, 0, 0], c2.kv_cache[0, 1, 0], k2.unsqueeze(2), v2.unsqueeze(2), c2.page_table))
+        rings.append((c2.kv_cache[0, 0, 0], c2.kv_cache[0, 1, 0], k2.unsqueeze(2), v2.unsqueeze(2), c2.page_table,
+                      torch.empty_like(out)))
     turn = [0]
 
     def do_append_cold():
-        rk, rv, sk, sv, table = rings[turn[0] % len(rings)]
+        rk, rv, sk, sv, table, _ = rings[turn[0] % len(rings)]
         turn[0] += 1
         ops.kv_append(rk, rv, sk, sv, table, flat_b, flat_p, P, clamp_negative=False)
+
+    def do_gather_cold():
+        rk, _, _, _, table, o = rings[turn[0] % len(rings)]
+        turn[0] += 1
+        ops.kv_gather(rk, table, slots, lens, P, T, out=o)
 
     for _ in range(len(rings)):
         do_append_cold()
     ms_cold = event_ms(do_append_cold, 3 * len(rings))
+    ms_g_cold = event_ms(do_gather_cold, 3 * len(rings))
     del rings
 
     # QK norm + rotary embedding + insert in one launch (reference model.py:110-119 + the append):
@@ -503,7 +511,9 @@ def append_gather_rates(steps: int = 20, T: int = 32768, H: int = 16, D: int = 1
             "kv_append_cold_frac_of_peak": bytes_a / (ms_cold * 1e-3) / 1e9 / HBM_PEAK_GBPS,
             "kv_append_by_tokens": sweep,
             "kv_gather_ms": ms_g, "kv_gather_gbps": bytes_g / (ms_g * 1e-3) / 1e9,
-            "kv_gather_frac_of_peak": bytes_g / (ms_g * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+            "kv_gather_frac_of_peak": bytes_g / (ms_g * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "kv_gather_cold_ms": ms_g_cold, "kv_gather_cold_gbps": bytes_g / (ms_g_cold * 1e-3) / 1e9,
+            "kv_gather_cold_frac_of_peak": bytes_g / (ms_g_cold * 1e-3) / 1e9 / HBM_PEAK_GBPS}
 
 
 def prefill_rate(steps: int = 10, name: str = "cfg3") -> dict:
