@@ -36,7 +36,10 @@ int fp::compute_units() {
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
   if (cached[dev] == 0) {
     int n = 0;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+      (void)hipGetLastError();
+      n = 256;
+    }
     cached[dev] = n;
   }
   return cached[dev];

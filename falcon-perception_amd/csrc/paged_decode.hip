@@ -825,9 +825,10 @@ int resident_workgroups() {
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
   if (cached[dev] == 0) {
     int per_cu = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kThreads, 0) != hipSuccess || per_cu <= 0)
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kThreads, 0) != hipSuccess || per_cu <= 0) {
+      (void)hipGetLastError();  // not an error of the launch that follows: the launch goes split by split
       cached[dev] = -1;
-    else
+    } else
       cached[dev] = per_cu * fp::compute_units();
   }
   return cached[dev] > 0 ? cached[dev] : 0;

@@ -113,3 +113,44 @@ def test_prefill_random(seed):
     atol, rtol = TOL[dtype]
     np.testing.assert_allclose(f64(out), eo, atol=atol, rtol=rtol)
     np.testing.assert_allclose(f64(lse), el, atol=max(atol * 0.1, 1e-4), rtol=rtol)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_decode_random_large_launches(seed):
+    """Many sequences and small splits, so that the launch has more workgroups than the GPU holds at once
+    (16-bit dtypes then take the even cut over the flattened contexts): batch sizes that are no multiple
+    of 64, empty and masked-out sequences, every page size and head grouping of `draw`."""
+    rng, P, D, G, Hc, dtype = draw(200 + seed, [torch.bfloat16, torch.float16, torch.float32])
+    Hc = int(rng.choice([4, 8]))
+    B = int(rng.integers(90, 260))
+    lens = [int(x) for x in rng.integers(0, 400, B)]
+    lens[int(rng.integers(B))] = 0
+    n_pages = sum(-(-(L + 1) // P) for L in lens) + 4
+    st = PagedState(300 + seed, n_pages=n_pages, page_size=P, max_batch=B + 2, Hc=Hc, D=D, dtype=dtype)
+    for L in lens:
+        st.add_sequence(L + 1)
+    st.lens = lens
+    st.prefill_random()
+    k1, v1 = randn(st.gen, (B, Hc, 1, D), dtype), randn(st.gen, (B, Hc, 1, D), dtype)
+    q = randn(st.gen, (B, Hc * G, 1, D), dtype)
+    pos = torch.tensor(lens, dtype=torch.int32)
+    bidx = torch.tensor(st.slots, dtype=torch.int64, device=DEV)
+    masked = int(rng.integers(B))
+    bidx[masked] = -1  # not a cache slot: out 0, lse -inf, nothing appended
+    pk, pv = st.pool_planes()
+    max_ctx = 448
+    before = st.cache.kv_cache.clone()
+    out, lse = ops.paged_decode(q.to(DEV), pk, pv, st.cache.page_table, bidx, pos.to(DEV), P, max_ctx,
+                                split_tokens=64, k_new=k1.to(DEV), v_new=v1.to(DEV))
+    keep = [i for i in range(B) if i != masked]
+    want = before.cpu().clone()
+    wv = want.view(torch.int16 if dtype != torch.float32 else torch.int32).numpy()
+    O.append_decode(wv, 0, bits(k1)[keep], bits(v1)[keep], st.mirror.page_table, np.array(st.slots)[keep],
+                    pos.view(B, 1).numpy()[keep], P)
+    assert np.array_equal(bits(st.cache.kv_cache), wv)
+    eo, el = O.decode_attention(f64(q)[keep], f64(pk), f64(pv), st.mirror.page_table, [st.slots[i] for i in keep],
+                                pos.numpy()[keep], P)
+    atol, rtol = TOL[dtype]
+    np.testing.assert_allclose(f64(out)[keep], eo, atol=atol, rtol=rtol)
+    np.testing.assert_allclose(f64(lse)[keep], el, atol=max(atol * 0.1, 2e-5), rtol=rtol)
+    assert not f64(out)[masked].any() and np.isneginf(f64(lse)[masked]).all()
