@@ -266,10 +266,11 @@ __device__ __forceinline__ void fold_rows(const v4u (&kreg)[GK][U], const v4u (&
 constexpr int decode_loads_in_flight(int G, bool per_head_k) { return per_head_k && G >= 4 ? 4 : 8; }
 
 // Four workgroups per CU instead of three (at most 128 registers) where the kernel fits without spilling:
-// one query head per cache head, and two in fp32 (the 16-bit kernels keep twice the elements per lane).
-template <typename E, int D, int G, bool kPerHeadK>
+// one query head per cache head, and two in fp32 (the 16-bit kernels keep twice the elements per lane).  Not for
+// the even cut, which runs two workgroups per CU.
+template <typename E, int D, int G, bool kPerHeadK, bool kFlat>
 constexpr int decode_waves_per_simd() {
-  return (!kPerHeadK && (G == 1 || (G == 2 && sizeof(typename E::type) == 4))) ? 4 : 1;
+  return (!kFlat && !kPerHeadK && (G == 1 || (G == 2 && sizeof(typename E::type) == 4))) ? 4 : 1;
 }
 
 // Even cut of a launch (kFlat): the contexts of the launch, each rounded up to 64 tokens, are laid end
@@ -325,7 +326,7 @@ __device__ __forceinline__ int flat_chunk_len(int total, int n_chunks) {
 }
 
 template <typename E, int D, int G, bool kDirect, bool kAligned, bool kPerHeadK = false, bool kFlat = false>
-__global__ __launch_bounds__(kThreads, (decode_waves_per_simd<E, D, G, kPerHeadK>())) void paged_decode_kernel(const DecodeArgs a) {
+__global__ __launch_bounds__(kThreads, (decode_waves_per_simd<E, D, G, kPerHeadK, kFlat>())) void paged_decode_kernel(const DecodeArgs a) {
   constexpr int EPL = E::kEpl;          // elements per lane
   constexpr int TPR = D / EPL;          // lanes per row
   constexpr int RPW = 64 / TPR;         // rows per wavefront load
@@ -848,15 +849,16 @@ void launch_decode(const DecodeArgs& a, int B, int phases, hipStream_t st) {
     else
       hipLaunchKernelGGL((paged_decode_kernel<E, D, G, true, false, kPerHeadK>), grid, dim3(kThreads), 0, st, a);
   } else {
-    // A 16-bit launch with more workgroups than the GPU holds at once is cut evenly instead: two chunks
+    // A launch with more workgroups than the GPU holds at once is cut evenly instead: two chunks
     // per CU, all of the same length, all resident from the start, so that every CU streams the same
     // number of rows (split by split, the CUs end up with loads 25 % apart at 64 sequences of 1 k to
     // 4 k tokens, and workgroups queue behind busy shader engines).  Measured at 64 sequences of 16 q /
     // 8 kv heads, bf16, % of 8 TB/s for the step with 1 / 2 / 3 / 4 chunks per CU and split by split:
     // D 128: 75.5 / 75.4 / 73.8 / 73.1 and 73.0; D 64: 67.2 / 68.3 / 68.1 / 63.7 and 67.1; 32 q heads:
-    // 63.9 / 70.6 / 64.2 / 67.9 and 67.2; 16-token pages: 70.0 / 74.4 / 73.9 / 68.9 and 72.6.  fp32 is
-    // faster split by split (D 128: 77.5 against 73.8 / 70.4 / 69.6 / 69.2) and stays so.  The even cut
-    // needs the lengths of at most kFlatMaxB sequences in LDS, a workspace row per (chunk + sequence),
+    // 63.9 / 70.6 / 64.2 / 67.9 and 67.2; 16-token pages: 70.0 / 74.4 / 73.9 / 68.9 and 72.6.  fp32 with
+    // two chunks per CU: D 128 80.7 against 78.4 split by split, D 64 76.9 against 76.1, 32 q heads 77.4
+    // against 73.4 (the even-cut kernels are not held to 128 registers: two workgroups per CU do not need
+    // it, and in fp32 it made them spill).  The even cut needs the lengths of at most kFlatMaxB sequences in LDS, a workspace row per (chunk + sequence),
     // and chunks within the page-id table.
     int n_chunks = 0;
     {
@@ -864,7 +866,7 @@ void launch_decode(const DecodeArgs& a, int B, int phases, hipStream_t st) {
                                    : resident_workgroups<E, D, G, false, kPerHeadK>();
       const int64_t wgs = static_cast<int64_t>(a.Hc) * B * a.n_splits;
       const int chunks = 2 * fp::compute_units() / a.Hc;
-      if (sizeof(typename E::type) == 2 && chunks >= 1 && wgs > resident && B <= kFlatMaxB &&
+      if (chunks >= 1 && wgs > resident && B <= kFlatMaxB &&
           static_cast<int64_t>(B) * (a.max_context + 64) < (1ll << 30) &&  // positions on the flat axis are int chunks + B <= static_cast<int64_t>(B) * a.n_splits &&
           (static_cast<int64_t>(B) * a.max_context / chunks + 128) / a.pd.page_size + 2 <= kMaxSplitPages)
         n_chunks = chunks;

@@ -187,7 +187,7 @@ int fp_paged_decode(const void* q, int64_t q_stride_b, int64_t q_stride_h,
  * leaves, per (sequence, query head, piece of the context), the unnormalised accumulator,
  * running maximum and denominator in the workspace (log2 units); the merge pass combines
  * them into out and lse.  The pieces are the splits of split_tokens tokens
- * ([B, Hq, n_splits, D] floats followed by [B, Hq, n_splits, 2] floats), except that a 16-bit
+ * ([B, Hq, n_splits, D] floats followed by [B, Hq, n_splits, 2] floats), except that a
  * launch of more workgroups than the GPU holds at once is cut into equal chunks of the
  * contexts laid end to end (rows (chunk + sequence) * Hq + head of [rows, D] and [rows, 2]
  * floats): the layout is a matter between the two passes.  For callers that time or

@@ -118,7 +118,7 @@ def test_prefill_random(seed):
 @pytest.mark.parametrize("seed", range(8))
 def test_decode_random_large_launches(seed):
     """Many sequences and small splits, so that the launch has more workgroups than the GPU holds at once
-    (16-bit dtypes then take the even cut over the flattened contexts): batch sizes that are no multiple
+    (the launch then takes the even cut over the flattened contexts): batch sizes that are no multiple
     of 64, empty and masked-out sequences, every page size and head grouping of `draw`."""
     rng, P, D, G, Hc, dtype = draw(200 + seed, [torch.bfloat16, torch.float16, torch.float32])
     Hc = int(rng.choice([4, 8]))
