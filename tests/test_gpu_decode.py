@@ -331,3 +331,26 @@ def test_a_launch_larger_than_the_gpu_is_cut_evenly(dtype, D, P, G):
         g.replay()
         torch.cuda.synchronize()
         assert torch.equal(out_g, out) and torch.equal(lse_g, lse)
+
+
+@pytest.mark.parametrize("B,ctx", [(50, 128), (100, 128), (97, 192), (200, 256)])
+def test_no_pass_writes_outside_the_workspace_it_asked_for(B, ctx):
+    """Launches around the point where the even cut takes over (8 heads x B sequences x 2 to 4 splits
+    against the workgroups the GPU holds at once): the even cut needs a workspace row per (chunk +
+    sequence) and must leave the launch alone where the rows asked for split by split would not hold them.
+    The workspace sits inside a larger buffer whose remainder must come back untouched."""
+    dtype, D, P, Hc, G, split = torch.bfloat16, 128, 32, 8, 2, 64
+    st = PagedState(35, n_pages=B * (-(-ctx // P)) + 8, page_size=P, max_batch=B + 2, Hc=Hc, D=D, dtype=dtype)
+    lens = torch.randint(1, ctx, (B,), generator=st.gen).tolist()
+    for L in lens:
+        st.add_sequence(L)
+    st.prefill_random()
+    q = randn(st.gen, (B, Hc * G, 1, D), dtype)
+    pos = torch.tensor(lens, dtype=torch.int32) - 1
+    need = ops.decode_workspace_bytes(B, Hc * G, D, ctx, split)
+    guard = 1 << 20
+    buf = torch.full((need + guard,), 0x5A, dtype=torch.uint8, device=DEV)
+    out, lse = run_decode(st, q, pos, workspace=buf[:need], split_tokens=split, max_context=ctx)
+    assert bool((buf[need:] == 0x5A).all())
+    eo, el = oracle_decode(st, q, pos)
+    assert_close(out, lse, eo, el, dtype)
