@@ -869,7 +869,7 @@ void launch_decode(const DecodeArgs& a, int B, int phases, hipStream_t st) {
       const bool rows_fit = chunks + B <= static_cast<int64_t>(B) * a.n_splits;  // workspace rows: one per (chunk + sequence)
       const bool positions_fit = static_cast<int64_t>(B) * (a.max_context + 64) < (1ll << 30);  // the flat axis is int
       if (chunks >= 1 && wgs > resident && B <= kFlatMaxB && rows_fit && positions_fit &&
-          (static_cast<int64_t>(B) * a.max_context / chunks + 128) / a.pd.page_size + 2 <= kMaxSplitPages)
+          (static_cast<int64_t>(B) * (a.max_context + 64) / chunks + 128) / a.pd.page_size + 2 <= kMaxSplitPages)
         n_chunks = chunks;
     }
     DecodeArgs af = a;
