@@ -105,3 +105,21 @@ def test_large_launches_ask_for_no_workspace():
     assert ops.prefill_workspace_bytes(512, 16, 8, 128, torch.bfloat16) == 8 * 512 * 16 * 130 * 4
     with pytest.raises(RuntimeError, match="fp_paged_prefill_workspace_bytes"):
         ops.prefill_workspace_bytes(512, 12, 8, 128, torch.bfloat16)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=str)
+def test_the_passes_stay_inside_the_workspace_they_asked_for(dtype):
+    D, P = 128, 64
+    st, q, bidx, lim = make_case(dtype, D, 2, P, lens=[333, 900, 70], pads=[1, 0, 2])
+    pk, pv = st.pool_planes()
+    need = ops.prefill_workspace_bytes(q.shape[2], q.shape[1], pk.shape[0], D, dtype)
+    assert need > 0
+    guard = 1 << 20
+    for nbytes in (need, need // 2, need // 4 + 16):  # what the library asked for, and less (coarser cuts)
+        buf = torch.full((nbytes + guard,), 0x5A, dtype=torch.uint8, device=DEV)
+        out, lse = ops.paged_prefill(q.to(DEV), pk, pv, st.cache.page_table, bidx, lim, P, workspace=buf[:nbytes])
+        assert bool((buf[nbytes:] == 0x5A).all())
+        atol, rtol = TOL[dtype]
+        eo, el = O.prefill_attention_paged(f64(q), f64(pk), f64(pv), st.mirror.page_table, bidx.cpu().numpy(), None,
+                                           lim.cpu().numpy(), P)
+        np.testing.assert_allclose(f64(out), eo, atol=atol, rtol=rtol)
