@@ -68,6 +68,6 @@ int prefill_mfma_f32(const void* q, int64_t q_stride_row, int64_t q_stride_h, co
 // Key shares the prefill kernel of `dtype` cuts a launch of `wgs` workgroups into on the current device
 // (1 .. 8), and the workspace bytes `shares` of them need (paged_prefill.hip)
 int prefill_key_shares(int64_t wgs, int dtype);
-int64_t prefill_share_bytes(int shares, int Lq, int Hq, int D);
+int64_t prefill_share_bytes(int shares, int Lq, int Hq, int D, int elem_bytes);
 
 }  // namespace fp

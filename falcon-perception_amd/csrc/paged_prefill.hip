@@ -72,7 +72,9 @@ struct PrefillArgs {
   int n_tiles;   // query tiles
   // key split: grid z = n_key_splits workgroups share a query tile, each taking an equal share of every
   // run's key tiles and leaving unnormalised partial results for the merge pass
-  float* ws_acc;  // [n_key_splits, Lq, Hq, D]
+  // key shares: a share's result for a row, normalised by its own denominator, in the model dtype (half
+  // the bytes of fp32 partials; the merge pass is bound by this traffic), with its maximum and denominator
+  short* ws_acc;  // [n_key_splits, Lq, Hq, D] elements of the model dtype
   float* ws_ml;   // [n_key_splits, Lq, Hq, 2]: running maximum (log2 units), denominator
 };
 
@@ -90,6 +92,7 @@ struct BF16 {
     return __builtin_bit_cast(uint32_t, v);
   }
   static __device__ __forceinline__ float round(float x) { return static_cast<float>(static_cast<__bf16>(x)); }
+  static __device__ __forceinline__ float to_float(short x) { return static_cast<float>(__builtin_bit_cast(__bf16, x)); }
 };
 struct F16 {
   using vec8 = f16x8;
@@ -105,6 +108,7 @@ struct F16 {
     return __builtin_bit_cast(uint32_t, v);
   }
   static __device__ __forceinline__ float round(float x) { return static_cast<float>(static_cast<_Float16>(x)); }
+  static __device__ __forceinline__ float to_float(short x) { return static_cast<float>(__builtin_bit_cast(_Float16, x)); }
 };
 
 constexpr f32x16 kZero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
@@ -268,7 +272,7 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
         if (gridDim.z > 1) {  // an empty share; the merge pass then writes out = 0, lse = -inf
           const int64_t p = (static_cast<int64_t>(blockIdx.z) * a.Lq + row[mb]) * a.Hq + hq;
 #pragma unroll
-          for (int c = 0; c < D / 8; ++c) *reinterpret_cast<f32x4*>(a.ws_acc + p * D + half * (D / 2) + c * 4) = f32x4{0, 0, 0, 0};
+          for (int c = 0; c < D / 8; ++c) *reinterpret_cast<uint2*>(a.ws_acc + p * D + half * (D / 2) + c * 4) = uint2{0, 0};
           if (half == 0) *reinterpret_cast<float2*>(a.ws_ml + p * 2) = float2{-INFINITY, 0.f};
           continue;
         }
@@ -617,13 +621,14 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
       if (gridDim.z > 1) {
         // one of several key shares: the unnormalised state goes to the merge pass
         const int64_t p = (static_cast<int64_t>(blockIdx.z) * a.Lq + row[mb]) * a.Hq + hq;
-        float* po = a.ws_acc + p * D;
+        short* po = a.ws_acc + p * D;
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll
           for (int i4 = 0; i4 < 4; ++i4)
-            *reinterpret_cast<f32x4*>(po + db * 32 + i4 * 8 + half * 4) =
-                f32x4{o_acc[mb][db][i4 * 4], o_acc[mb][db][i4 * 4 + 1], o_acc[mb][db][i4 * 4 + 2], o_acc[mb][db][i4 * 4 + 3]};
+            *reinterpret_cast<uint2*>(po + db * 32 + i4 * 8 + half * 4) =
+                uint2{E::pack2(o_acc[mb][db][i4 * 4] * inv, o_acc[mb][db][i4 * 4 + 1] * inv),
+                      E::pack2(o_acc[mb][db][i4 * 4 + 2] * inv, o_acc[mb][db][i4 * 4 + 3] * inv)};
         if (half == 0) *reinterpret_cast<float2*>(a.ws_ml + p * 2) = float2{m_run[mb], l_tot};
         continue;
       }
@@ -652,8 +657,8 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
 }
 
 // ---- merge of the key shares ----
-// One wavefront per (query row, query head): combines the shares' unnormalised accumulators with
-// their running maxima and denominators, applies the sink gate, stores out and lse.
+// One wavefront per (query row, query head): combines the shares' results, each weighted by its
+// denominator at the common maximum, applies the sink gate, stores out and lse.
 constexpr int kMergeRows = 4;  // (row, head) pairs per workgroup
 
 template <typename E, int D>
@@ -672,8 +677,13 @@ __global__ __launch_bounds__(kMergeRows * 64) void paged_prefill_merge_kernel(co
     const int64_t p = s * share_stride + item;
     m_s[s] = on ? a.ws_ml[p * 2] : -INFINITY;
     l_s[s] = on ? a.ws_ml[p * 2 + 1] : 0.f;
-#pragma unroll
-    for (int e = 0; e < EPL; ++e) acc_s[s][e] = on ? a.ws_acc[p * D + lane * EPL + e] : 0.f;
+    if (EPL == 2) {
+      const uint32_t w = on ? *reinterpret_cast<const uint32_t*>(a.ws_acc + p * D + lane * 2) : 0u;
+      acc_s[s][0] = E::to_float(static_cast<short>(w & 0xffffu));
+      acc_s[s][EPL - 1] = E::to_float(static_cast<short>(w >> 16));
+    } else {
+      acc_s[s][0] = on ? E::to_float(a.ws_acc[p * D + lane]) : 0.f;
+    }
   }
   float mn = -INFINITY;
 #pragma unroll
@@ -684,8 +694,8 @@ __global__ __launch_bounds__(kMergeRows * 64) void paged_prefill_merge_kernel(co
   for (int e = 0; e < EPL; ++e) num[e] = 0.f;
 #pragma unroll
   for (int s = 0; s < kBatch; ++s) {
-    const float wgt = fast_exp2(m_s[s] - ms);  // 0 for a share that saw no key
-    den += l_s[s] * wgt;
+    const float wgt = l_s[s] * fast_exp2(m_s[s] - ms);  // 0 for a share that saw no key
+    den += wgt;
 #pragma unroll
     for (int e = 0; e < EPL; ++e) num[e] += acc_s[s][e] * wgt;
   }
@@ -717,8 +727,9 @@ int key_shares_for(int64_t wgs, int dtype) {
   return static_cast<int>(n < 1 ? 1 : n > kMaxKeyShares ? kMaxKeyShares : n);
 }
 
-int64_t share_bytes(int shares, int Lq, int Hq, int D) {
-  return shares <= 1 ? 0 : static_cast<int64_t>(shares) * Lq * Hq * (D + 2) * static_cast<int64_t>(sizeof(float));
+// workspace of `shares` key shares: per row and head D results of elem bytes, and two floats
+int64_t share_bytes(int shares, int Lq, int Hq, int D, int elem) {
+  return shares <= 1 ? 0 : static_cast<int64_t>(shares) * Lq * Hq * (static_cast<int64_t>(D) * elem + 8);
 }
 
 template <typename E, int D, int G>
@@ -727,10 +738,10 @@ void launch_group(const PrefillArgs& a0, void* workspace, int64_t workspace_byte
   constexpr int BM = (kWaves / G) * 32;
   a.n_tiles = (a.Lq + BM - 1) / BM;
   int shares = workspace ? key_shares_for(static_cast<int64_t>(a.Hc) * a.n_tiles, FP_DTYPE_BF16) : 1;  // f16 alike
-  while (shares > 1 && share_bytes(shares, a.Lq, a.Hq, D) > workspace_bytes) --shares;  // what the workspace holds
+  while (shares > 1 && share_bytes(shares, a.Lq, a.Hq, D, 2) > workspace_bytes) --shares;  // what the workspace holds
   if (shares > 1) {
-    a.ws_acc = static_cast<float*>(workspace);
-    a.ws_ml = a.ws_acc + static_cast<int64_t>(shares) * a.Lq * a.Hq * D;
+    a.ws_ml = static_cast<float*>(workspace);
+    a.ws_acc = reinterpret_cast<short*>(a.ws_ml + static_cast<int64_t>(shares) * a.Lq * a.Hq * 2);
   }
   dim3 grid(a.Hc, a.n_tiles, shares);
   if (a.pd.shift >= 0)
@@ -821,8 +832,9 @@ extern "C" int64_t fp_paged_prefill_workspace_bytes(int32_t Lq, int32_t Hq, int3
   if (dtype != FP_DTYPE_BF16 && dtype != FP_DTYPE_F16 && dtype != FP_DTYPE_F32)
     return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill_workspace_bytes: unknown dtype %d", dtype);
   const int bm = (kWaves / g) * 32;
-  return share_bytes(key_shares_for(static_cast<int64_t>(Hc) * ((Lq + bm - 1) / bm), dtype), Lq, Hq, D);
+  return share_bytes(key_shares_for(static_cast<int64_t>(Hc) * ((Lq + bm - 1) / bm), dtype), Lq, Hq, D,
+                     fp::elem_bytes(dtype));
 }
 
 int fp::prefill_key_shares(int64_t wgs, int dtype) { return key_shares_for(wgs, dtype); }
-int64_t fp::prefill_share_bytes(int shares, int Lq, int Hq, int D) { return share_bytes(shares, Lq, Hq, D); }
+int64_t fp::prefill_share_bytes(int shares, int Lq, int Hq, int D, int elem) { return share_bytes(shares, Lq, Hq, D, elem); }

@@ -464,7 +464,7 @@ void launch_group(const Args& a0, void* workspace, int64_t workspace_bytes, hipS
   constexpr int BM = (kWaves / G) * 32;
   a.n_tiles = (a.Lq + BM - 1) / BM;
   int shares = workspace ? fp::prefill_key_shares(static_cast<int64_t>(a.Hc) * a.n_tiles, FP_DTYPE_F32) : 1;
-  while (shares > 1 && fp::prefill_share_bytes(shares, a.Lq, a.Hq, D) > workspace_bytes) --shares;
+  while (shares > 1 && fp::prefill_share_bytes(shares, a.Lq, a.Hq, D, 4) > workspace_bytes) --shares;
   if (shares > 1) {
     a.ws_acc = static_cast<float*>(workspace);
     a.ws_ml = a.ws_acc + static_cast<int64_t>(shares) * a.Lq * a.Hq * D;

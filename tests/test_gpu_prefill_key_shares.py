@@ -66,7 +66,7 @@ def test_a_smaller_workspace_gives_a_coarser_cut_and_the_same_answer():
     pk, pv = st.pool_planes()
     Hq, Lq = q.shape[1], q.shape[2]
     need = ops.prefill_workspace_bytes(Lq, Hq, pk.shape[0], D, dtype)
-    two_shares = 2 * Lq * Hq * (D + 2) * 4
+    two_shares = 2 * Lq * Hq * (D * 2 + 8)  # per row and head: D bf16 results, maximum and denominator
     assert need > two_shares
     full, _ = ops.paged_prefill(q.to(DEV), pk, pv, st.cache.page_table, bidx, lim, P,
                                 workspace=torch.empty(need, dtype=torch.uint8, device=DEV))
@@ -102,7 +102,7 @@ def test_large_launches_ask_for_no_workspace():
     rows = 128 * (cus // 8)
     assert ops.prefill_workspace_bytes(rows, 16, 8, 128, torch.bfloat16) == 0
     assert ops.prefill_workspace_bytes(rows, 16, 8, 128, torch.float32) == 4 * rows * 16 * 130 * 4
-    assert ops.prefill_workspace_bytes(512, 16, 8, 128, torch.bfloat16) == 8 * 512 * 16 * 130 * 4
+    assert ops.prefill_workspace_bytes(512, 16, 8, 128, torch.bfloat16) == 8 * 512 * 16 * (128 * 2 + 8)
     with pytest.raises(RuntimeError, match="fp_paged_prefill_workspace_bytes"):
         ops.prefill_workspace_bytes(512, 12, 8, 128, torch.bfloat16)
 
