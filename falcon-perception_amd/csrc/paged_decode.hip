@@ -9,7 +9,10 @@
 // HBM-bound: every cached K and V row of every sequence is read exactly once.
 //   grid  = (cache heads, batch, splits); a workgroup of 4 wavefronts owns one
 //           (sequence, cache head, token range) and serves all G = Hq / Hc query
-//           heads of that cache head from a single read of K and V.
+//           heads of that cache head from a single read of K and V.  A launch
+//           larger than the GPU holds at once runs as (cache heads, chunks)
+//           instead: the contexts laid end to end and cut into equal chunks, a
+//           workgroup working through the sequences its chunk touches.
 //   loads = a row (D elements) is covered by TPR = D * elem / 16 lanes holding
 //           16 bytes each, so a wavefront load instruction moves 64 / TPR whole
 //           rows, contiguous inside a page; U such loads of K and of V are in
