@@ -9,6 +9,19 @@
 // with q's span id, which ends at the first k > q that is not inside or is a soi.
 // So row q may see keys up to  row_hi[q] = inside[q] ? that k : q + 1.
 //
+// That closed form equals the reference's mask exactly when every span opens and closes
+// inside one document of the packed row (what the reference's engine packs,
+// paged_inference.py:637-672: whole sequences, each padded to 128).  Two inputs break it and
+// are reported through `status` instead of being answered wrongly:
+//   bit 0  an eoi with no span open -- the chunk starts inside an image span whose soi lies in
+//          an earlier chunk.  The caller can declare that with `open_at_start[slot] != 0`: the
+//          first row of that slot's run then counts as preceded by a soi, and the rows up to
+//          the eoi get the eoi's index as their limit (every earlier key of the span is below
+//          the row anyway, so one limit per row still is the whole mask);
+//   bit 1  a span still open where the document changes or the row ends -- its rows would need
+//          keys of another document (what the reference's global counts would allow) or keys
+//          that are not in the cache yet.
+//
 // One workgroup scans the packed row: each thread owns a contiguous chunk, the
 // chunk totals are combined with an LDS prefix sum (forward) and an LDS suffix
 // minimum (backward).  L is at most 65536 tokens, the work is a few microseconds.
@@ -19,14 +32,29 @@ namespace {
 constexpr int kThreads = 1024;
 constexpr int kMaxL = 65536;
 
-__global__ __launch_bounds__(kThreads) void hybrid_row_limits_kernel(const int64_t* __restrict__ ids, int L,
+// a soi counted in front of token k: k starts a run of a slot declared open
+__device__ __forceinline__ bool virtual_soi(const int64_t* __restrict__ docs, const uint8_t* __restrict__ open_at_start,
+                                            int max_batch, int k) {
+  if (!docs || !open_at_start) return false;
+  const int64_t d = docs[k];
+  if (k > 0 && docs[k - 1] == d) return false;
+  return d >= 0 && d < max_batch && open_at_start[d] != 0;
+}
+
+__global__ __launch_bounds__(kThreads) void hybrid_row_limits_kernel(const int64_t* __restrict__ ids,
+                                                                     const int64_t* __restrict__ docs,
+                                                                     const uint8_t* __restrict__ open_at_start,
+                                                                     int max_batch, int L,
                                                                      int64_t soi, int64_t eoi,
-                                                                     int32_t* __restrict__ row_hi) {
+                                                                     int32_t* __restrict__ row_hi,
+                                                                     int32_t* __restrict__ status) {
   __shared__ int s_soi[kThreads];
   __shared__ int s_eoi[kThreads];
   __shared__ int s_next[kThreads];
+  __shared__ int s_flags;
 
   const int tid = threadIdx.x;
+  if (tid == 0) s_flags = 0;
   const int per = (L + kThreads - 1) / kThreads;
   const int lo = min(tid * per, L);
   const int hi = min(lo + per, L);
@@ -34,7 +62,7 @@ __global__ __launch_bounds__(kThreads) void hybrid_row_limits_kernel(const int64
   int n_soi = 0, n_eoi = 0;
   for (int k = lo; k < hi; ++k) {
     const int64_t id = ids[k];
-    n_soi += id == soi;
+    n_soi += (id == soi) + virtual_soi(docs, open_at_start, max_batch, k);
     n_eoi += id == eoi;
   }
   s_soi[tid] = n_soi;
@@ -54,16 +82,22 @@ __global__ __launch_bounds__(kThreads) void hybrid_row_limits_kernel(const int64
 
   // first index in this chunk that ends a span (not inside, or a soi), L if none
   int first_end = L;
+  int flags = 0;
   {
     int o = base_soi, c = base_eoi;
     for (int k = lo; k < hi; ++k) {
       const int64_t id = ids[k];
-      o += id == soi;
+      const bool virt = virtual_soi(docs, open_at_start, max_batch, k);
+      o += (id == soi) + virt;
       c += id == eoi;
-      const bool ends = !(o - c > 0) || id == soi;
+      const bool ends = !(o - c > 0) || id == soi || virt;
       if (ends && first_end == L) first_end = k;
+      if (o - c < 0) flags |= 1;
+      const bool run_ends = k == L - 1 || (docs && docs[k + 1] != docs[k]);
+      if (run_ends && o - c > 0) flags |= 2;
     }
   }
+  if (flags) atomicOr(&s_flags, flags);
   s_next[tid] = first_end;
   __syncthreads();
   // inclusive suffix minimum over chunks
@@ -80,22 +114,28 @@ __global__ __launch_bounds__(kThreads) void hybrid_row_limits_kernel(const int64
   for (int k = hi - 1; k >= lo; --k) {
     const int64_t id = ids[k];
     const bool inside = o - c > 0;
+    const bool virt = virtual_soi(docs, open_at_start, max_batch, k);
     row_hi[k] = inside ? next_end : k + 1;
-    if (!inside || id == soi) next_end = k;
-    o -= id == soi;
+    if (!inside || id == soi || virt) next_end = k;
+    o -= (id == soi) + virt;
     c -= id == eoi;
   }
+  if (tid == 0 && status) *status = s_flags;  // every atomicOr lies before the barriers of the suffix scan
 }
 
 }  // namespace
 
-extern "C" int fp_hybrid_row_limits(const int64_t* input_ids, int32_t L, int64_t soi_id, int64_t eoi_id,
-                                    int32_t* row_hi, void* stream) {
+extern "C" int fp_hybrid_row_limits(const int64_t* input_ids, const int64_t* batch_idx,
+                                    const uint8_t* open_at_start, int32_t max_batch, int32_t L,
+                                    int64_t soi_id, int64_t eoi_id, int32_t* row_hi, int32_t* status,
+                                    void* stream) {
   if (L < 0) return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_hybrid_row_limits: negative length");
   if (L > kMaxL) return fp::fail(FP_ERR_UNSUPPORTED, "fp_hybrid_row_limits: L=%d exceeds %d", L, kMaxL);
   if (L == 0) return FP_OK;
   if (!input_ids || !row_hi) return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_hybrid_row_limits: null pointer");
+  if (open_at_start && (!batch_idx || max_batch <= 0))
+    return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_hybrid_row_limits: open_at_start needs batch_idx and max_batch");
   hipLaunchKernelGGL(hybrid_row_limits_kernel, dim3(1), dim3(kThreads), 0, static_cast<hipStream_t>(stream),
-                     input_ids, L, soi_id, eoi_id, row_hi);
+                     input_ids, batch_idx, open_at_start, max_batch, L, soi_id, eoi_id, row_hi, status);
   return fp::check_launch("fp_hybrid_row_limits");
 }

@@ -113,7 +113,8 @@ class HybridPrefillMask:
     `paged_attention.py:353-359`).
     """
 
-    def __init__(self, cache, batch_idx: Tensor, input_ids: Tensor, soi_id: int, eoi_id: int, block_size: int):
+    def __init__(self, cache, batch_idx: Tensor, input_ids: Tensor, soi_id: int, eoi_id: int, block_size: int,
+                 open_spans=None, validate: bool = True, row_hi: Tensor | None = None):
         self.cache = cache
         self.batch_idx = batch_idx
         self.input_ids = input_ids
@@ -122,19 +123,59 @@ class HybridPrefillMask:
         self.BLOCK_SIZE = (block_size, block_size)
         L = batch_idx.shape[1]
         self.seq_lengths = (L, L)
-        self.row_hi = ops.hybrid_row_limits(input_ids, soi_id, eoi_id)  # [L] int32, packed coordinates
+        if row_hi is None:  # [L] int32, packed coordinates
+            row_hi = self._limits_from_ids(open_spans, validate)
+        self.row_hi = row_hi
         self._arange = torch.arange(L, dtype=torch.int64, device=batch_idx.device)
-        self._step_key = None  # the step whose row limits are kept below
+        self._step_key = None  # (address, shape) of the positions whose row limits are kept below
+        self._step_layer = -1  # layer that asked last: a layer id that does not grow starts a new step
         self._row_limit = None
 
-    def row_limit(self, input_pos: Tensor) -> Tensor:
+    def _limits_from_ids(self, open_spans, validate: bool) -> Tensor:
+        """Run the row-limit kernel; reject packed rows whose hybrid mask is not one limit per row.
+
+        The reference's `or_masks(image_prefix, document_causal)` (`paged_attention.py:350-361`) counts
+        soi / eoi tokens over the whole packed row.  A span that is still open where the document changes
+        would let its rows see the next document, and a chunk that starts inside a span has no soi to
+        count: neither occurs in the reference's engine (whole sequences, `paged_inference.py:637-672`),
+        and both are refused here instead of being answered with a causal mask.  `open_spans` (cache
+        slots) declares the second case, which is then served: those rows are bidirectional up to the eoi.
+        Reading the kernel's status word waits for the stream once per prefill step."""
+        dev = self.batch_idx.device
+        open_at_start = None
+        if open_spans is not None:
+            flags = torch.zeros(self.cache.max_batch_size, dtype=torch.uint8)
+            for slot in open_spans:
+                flags[int(slot)] = 1
+            open_at_start = flags.to(dev)
+        status = torch.zeros(1, dtype=torch.int32, device=dev) if validate else None
+        row_hi = ops.hybrid_row_limits(self.input_ids, self.soi_id, self.eoi_id, self.batch_idx,
+                                       open_at_start, status)
+        if validate:
+            bits = int(status.item())
+            if bits & 1:
+                raise RuntimeError(
+                    "create_prefill_blockmask: an end-of-image token closes a span that was not opened in this "
+                    "packed row; a chunk that starts inside an image span must be declared with open_spans=[slot]")
+            if bits & 2:
+                raise RuntimeError(
+                    "create_prefill_blockmask: an image span is still open where batch_idx changes or the packed "
+                    "row ends; its rows would need keys of another sequence or keys that are not cached yet")
+        return row_hi
+
+    def row_limit(self, input_pos: Tensor, layer_id: int = 0) -> Tensor:
         """Logical key limit of each row: its position plus the reach of `row_hi` beyond the row.
-        Computed by the first layer of a step and kept for the others."""
-        key = (input_pos.data_ptr(), input_pos._version, tuple(input_pos.shape))
-        if key != self._step_key:
+
+        Computed by the first layer of a step and kept for the layers after it (`layer_id` growing over
+        the same positions tensor).  The key holds nothing that an inference tensor lacks: the reference's
+        engine builds `input_pos` under `torch.inference_mode()` (`paged_inference.py:646-675, 1331`),
+        where tensors carry no version counter."""
+        key = (input_pos.data_ptr(), tuple(input_pos.shape), input_pos.dtype)
+        if key != self._step_key or layer_id <= self._step_layer:
             reach = self.row_hi.to(torch.int64) - self._arange
             self._row_limit = (input_pos.reshape(-1) + reach).to(torch.int32)
             self._step_key = key
+        self._step_layer = layer_id
         return self._row_limit
 
 
@@ -228,7 +269,7 @@ def compiled_flex_attn_prefill(q: Tensor, k: Tensor, v: Tensor, score_mod=None, 
     pool_v = cache.kv_cache[step.layer_id, 1, 0]
     out, lse = ops.paged_prefill(
         q, pool_k, pool_v, cache.page_table, step.batch_idx,
-        block_mask.row_limit(step.input_pos), cache.page_size, scale=scale, sinks=sinks,
+        block_mask.row_limit(step.input_pos, step.layer_id), cache.page_size, scale=scale, sinks=sinks,
         workspace=cache.prefill_workspace(q.shape[2], q.shape[1], q.shape[3], pool_k.shape[0], q.dtype),
     )
     return _result(out, lse, return_aux, return_lse)

@@ -238,15 +238,37 @@ def paged_decode(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor, 
     return out, lse
 
 
-def hybrid_row_limits(input_ids: Tensor, soi_id: int, eoi_id: int) -> Tensor:
-    """Packed index one past the last key each packed row may see: max(q + 1, end of q's image span)."""
-    N.require_cuda(input_ids)
+def hybrid_row_limits(input_ids: Tensor, soi_id: int, eoi_id: int, batch_idx: Tensor | None = None,
+                      open_at_start: Tensor | None = None, status: Tensor | None = None) -> Tensor:
+    """Packed index one past the last key each packed row may see: max(q + 1, end of q's image span).
+
+    `batch_idx` [L] int64 names the document of every packed row, `open_at_start` [max_batch] uint8 the
+    slots whose rows begin inside an image span opened by an earlier chunk.  `status` (one int32, written
+    by the kernel) reports inputs for which one limit per row is not the reference's mask: bit 0 an eoi
+    with no span open, bit 1 a span open across a document boundary or the end of the row."""
+    N.require_cuda(input_ids, batch_idx, open_at_start, status)
     ids = input_ids.reshape(-1).contiguous()
     if ids.dtype != torch.int64:
         ids = ids.to(torch.int64)
-    out = torch.empty(ids.shape[0], dtype=torch.int32, device=ids.device)
-    rc = N.lib().fp_hybrid_row_limits(ids.data_ptr(), ids.shape[0], soi_id, eoi_id, out.data_ptr(),
-                                      N.stream_ptr(ids.device))
+    L = ids.shape[0]
+    docs_ptr = open_ptr = status_ptr = None
+    max_batch = 0
+    if batch_idx is not None:
+        batch_idx = batch_idx.reshape(-1).contiguous()
+        if batch_idx.dtype != torch.int64 or batch_idx.shape[0] != L:
+            raise RuntimeError("batch_idx must be int64 with one entry per packed row")
+        docs_ptr = batch_idx.data_ptr()
+    if open_at_start is not None:
+        if batch_idx is None or open_at_start.dtype != torch.uint8 or not open_at_start.is_contiguous():
+            raise RuntimeError("open_at_start must be a contiguous uint8 tensor and needs batch_idx")
+        open_ptr, max_batch = open_at_start.data_ptr(), open_at_start.numel()
+    if status is not None:
+        if status.dtype != torch.int32 or status.numel() != 1:
+            raise RuntimeError("status must hold one int32")
+        status_ptr = status.data_ptr()
+    out = torch.empty(L, dtype=torch.int32, device=ids.device)
+    rc = N.lib().fp_hybrid_row_limits(ids.data_ptr(), docs_ptr, open_ptr, max_batch, L, soi_id, eoi_id,
+                                      out.data_ptr(), status_ptr, N.stream_ptr(ids.device))
     N.check(rc, "fp_hybrid_row_limits")
     return out
 

@@ -295,10 +295,16 @@ class PagedKVCache(KVCacheBase):
         )
 
     def create_prefill_blockmask(self, batch_idx: Tensor, input_ids: Tensor, soi_id: int, eoi_id: int,
-                                 BLOCK_SIZE: int = 128) -> HybridPrefillMask:
-        """Mask of a packed prefill step: document-causal OR image-prefix (:343-362)."""
+                                 BLOCK_SIZE: int = 128, *, open_spans=None, validate: bool = True) -> HybridPrefillMask:
+        """Mask of a packed prefill step: document-causal OR image-prefix (:343-362).
+
+        `open_spans` and `validate` are not arguments of the reference: `open_spans` lists the cache slots
+        whose chunk begins inside an image span that an earlier chunk opened; with `validate` (default) a
+        packed row whose spans cross a document boundary, the end of the row, or start before it undeclared
+        raises RuntimeError (one host read of a device word) instead of yielding a wrong mask."""
         assert batch_idx.ndim == 2 and batch_idx.shape[0] == 1
-        return HybridPrefillMask(self, batch_idx, input_ids, soi_id, eoi_id, BLOCK_SIZE)
+        return HybridPrefillMask(self, batch_idx, input_ids, soi_id, eoi_id, BLOCK_SIZE,
+                                 open_spans=open_spans, validate=validate)
 
     # ------------------------------------------------ decode launch parameters
     def decode_split_tokens(self, B: int, Hc: int, max_context: int) -> int:

@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define FP_ABI_VERSION 3
+#define FP_ABI_VERSION 4
 
 /* element types of pool / q / k / v */
 #define FP_DTYPE_F32 0
@@ -294,13 +294,25 @@ int fp_qkv_norm_rope_append(const void* xq, const void* xk, const void* xv,
  * get_image_prefix_mask_mod (attention.py:75-96) by a closed form.
  *
  *   input_ids [L] int64 packed token ids, soi_id / eoi_id the span delimiters
+ *   batch_idx NULL, or [L] int64 cache slot of each packed row (the documents of the row); needed
+ *             for status bit 1 and for open_at_start
+ *   open_at_start  NULL, or [max_batch] bytes: slot s != 0 declares that the first row of slot s in
+ *             this packed row lies inside an image span whose soi was prefilled by an earlier chunk
+ *             (no counterpart in the reference, whose engine prefills whole sequences,
+ *             paged_inference.py:637-672); the rows up to the span's eoi then get the eoi's index
  *   row_hi    [L] int32 out: packed index one past the last key row q may see
  *             = max(q + 1, end of q's image span)
+ *   status    NULL, or one int32 out (written, not accumulated): 0 when row_hi is the reference's
+ *             mask; bit 0 = an eoi with no span open (a chunk that starts inside a span and was not
+ *             declared); bit 1 = a span still open where batch_idx changes or the row ends (its
+ *             rows would need keys of another document or keys not yet cached).  row_hi is then
+ *             not a usable mask and the caller must reject the step.
  * L <= 65536 (one workgroup scans the row).
  */
-int fp_hybrid_row_limits(const int64_t* input_ids, int32_t L,
+int fp_hybrid_row_limits(const int64_t* input_ids, const int64_t* batch_idx,
+                         const uint8_t* open_at_start, int32_t max_batch, int32_t L,
                          int64_t soi_id, int64_t eoi_id,
-                         int32_t* row_hi, void* stream);
+                         int32_t* row_hi, int32_t* status, void* stream);
 
 /*
  * Chunked-prefill attention over the paged cache under the hybrid mask, on the matrix

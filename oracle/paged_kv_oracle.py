@@ -313,6 +313,49 @@ def row_windows(batch_idx, input_ids, soi_id, eoi_id):
     return doc_start, hi
 
 
+def chunk_row_limits(batch_idx, input_ids, soi_id, eoi_id, open_slots=()):
+    """Row limits of a packed row of CHUNKS, with the conditions under which one limit per row is the mask.
+
+    The reference prefills whole sequences (paged_inference.py:637-672), so its mask (attention.py:75-96,
+    paged_attention.py:350-361) never meets a chunk that starts or ends inside an image span.  Per sequence
+    the mask is allowed(q, kv) = kv <= q OR (q and kv inside one span [soi, eoi)); for a chunk whose slot
+    is in `open_slots` the span was opened by an earlier chunk, so the rows before the chunk's first eoi
+    are inside it.  Walks every document run (stretch of equal batch_idx) with its own open/closed state.
+
+    Returns (hi[L] packed index one past the last visible key, status): status bit 0 = an eoi met with no
+    span open, bit 1 = a span still open at the end of a run (document change or end of the row).
+    """
+    docs = np.asarray(batch_idx).reshape(-1)
+    ids = np.asarray(input_ids).reshape(-1)
+    L = docs.shape[0]
+    hi = np.arange(1, L + 1, dtype=np.int64)
+    status = 0
+    k = 0
+    while k < L:
+        end = k
+        while end < L and docs[end] == docs[k]:
+            end += 1
+        depth = 1 if int(docs[k]) in set(int(s) for s in open_slots) else 0
+        start = k if depth else None  # first row of the span that is open now
+        for t in range(k, end):
+            if ids[t] == soi_id:
+                if depth > 0 and start is not None:  # a soi inside an open span starts a new span id
+                    hi[start:t] = np.maximum(hi[start:t], t)
+                depth += 1
+                start = t
+            elif ids[t] == eoi_id:
+                if depth <= 0:
+                    status |= 1
+                depth -= 1
+                if depth <= 0 and start is not None:
+                    hi[start:t] = np.maximum(hi[start:t], t)
+                    start = None
+        if depth > 0:
+            status |= 2
+        k = end
+    return hi, status
+
+
 # --------------------------------------------------------------------------
 # attention
 # --------------------------------------------------------------------------

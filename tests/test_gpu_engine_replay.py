@@ -1,7 +1,10 @@
 """GPU: the sequence of cache and attention calls the reference engine makes, replayed against
 the oracle.  Follows paged_inference.py: engine init (:321-352), graph capture with temporary
 one-page slots (:865-952), packed prefill (:608-733), decode steps through captured HIP graphs
-with padded batch buckets (:954-1031, :783-863), page growth and preemption (:1209-1238)."""
+with padded batch buckets (:954-1031, :783-863), page growth and preemption (:1209-1238).  As in
+the reference, the capture runs in the constructor, outside inference mode (:434-435), and everything
+`generate` does (admission, prefill, decode, growth, erase) runs under `torch.inference_mode()`
+(:1331; the server's loop likewise, server/engine_worker.py:126)."""
 
 import numpy as np
 import pytest
@@ -180,6 +183,12 @@ def tokens(n_text_before, n_img, n_text_after):
 def test_engine_call_sequence():
     eng = MiniEngine()
     eng.capture()
+    with torch.inference_mode():
+        generate(eng)
+
+
+def generate(eng):
+    assert torch.is_inference_mode_enabled()
     assert eng.cache.num_free_pages == N_PAGES - 1 and len(eng.cache.free_batch_idx) == MAX_BS - 1
 
     # step 1: prefill three sequences (image + text, text only, image at position 0)

@@ -203,3 +203,47 @@ def test_a_run_longer_than_the_tile_slot_table():
     eo, el = O.prefill_attention_paged(f64(q), f64(pk), f64(pv), st.mirror.page_table, bidx.numpy(),
                                        None, lim.numpy(), P)
     assert_close(out, lse, eo, el, dtype)
+
+
+@pytest.mark.parametrize("cut", [40, 101, 212])
+def test_chunk_boundary_inside_the_image_span(cut):
+    """A sequence of text + image block + text prefilled in two chunks whose boundary lies inside the
+    image span (rows 12 .. 211, eoi at 212).  The first chunk cannot be served (its span rows would need
+    keys that are not cached yet) and is refused; prefilled causally instead (K/V only matter), the second
+    chunk declared with open_spans equals the rows of the whole-sequence result."""
+    dtype = torch.bfloat16
+    Hc, G, D, P = 2, 2, 128, 64
+    ids = np.array([TXT] * 12 + [SOI] + [IMG + 1] * 4 + [IMG] * 195 + [EOI] + [TXT] * 60)
+    total = len(ids)
+    st = PagedState(21, n_pages=16, page_size=P, max_batch=4, Hc=Hc, D=D, dtype=dtype)
+    b = st.add_sequence(total)
+    bidx, pos = np.full(total, b), np.arange(total)
+    k = randn(st.gen, (1, Hc, total, D), dtype)
+    v = randn(st.gen, (1, Hc, total, D), dtype)
+    q = randn(st.gen, (1, Hc * G, total, D), dtype)
+    cache = st.cache
+    dev = lambda a: torch.from_numpy(a)[None].to(DEV)
+    if cut > 12:
+        with pytest.raises(RuntimeError, match="still open"):
+            cache.create_prefill_blockmask(dev(bidx[:cut]), dev(ids[:cut]), SOI, EOI)
+    cache.insert_kv(0, k[:, :, :cut].to(DEV), v[:, :, :cut].to(DEV), input_pos=dev(pos[:cut]), batch_idx=dev(bidx[:cut]))
+    if 12 < cut <= 212:
+        with pytest.raises(RuntimeError, match="open_spans"):
+            cache.create_prefill_blockmask(dev(bidx[cut:]), dev(ids[cut:]), SOI, EOI)
+    mask = cache.create_prefill_blockmask(dev(bidx[cut:]), dev(ids[cut:]), SOI, EOI, open_spans=[b])
+    K, V = cache.insert_kv(0, k[:, :, cut:].to(DEV), v[:, :, cut:].to(DEV), input_pos=dev(pos[cut:]),
+                           batch_idx=dev(bidx[cut:]))
+    out, aux = A.compiled_flex_attn_prefill(q[:, :, cut:].to(DEV), K, V, block_mask=mask, return_aux=AuxRequest(lse=True))
+    eo, el = O.prefill_attention_packed(f64(q), f64(k), f64(v), bidx[None], ids[None], SOI, EOI)
+    assert_close(out, aux.lse, eo[:, :, cut:], el[:, :, cut:], dtype)
+
+
+def test_span_open_across_a_document_boundary_is_refused():
+    ids = np.array([TXT] * 3 + [SOI] + [IMG] * 20 + [TXT] * 8 + [EOI] + [TXT] * 4)
+    bidx = np.array([1] * 24 + [2] * 13)
+    st = PagedState(22, n_pages=8, page_size=16, max_batch=4, Hc=1, D=64, dtype=torch.bfloat16)
+    dev = lambda a: torch.from_numpy(a)[None].to(DEV)
+    with pytest.raises(RuntimeError, match="still open"):
+        st.cache.create_prefill_blockmask(dev(bidx), dev(ids), SOI, EOI)
+    # unchecked, the call returns as before (the mask of such a row is unspecified)
+    st.cache.create_prefill_blockmask(dev(bidx), dev(ids), SOI, EOI, validate=False)

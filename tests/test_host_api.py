@@ -240,3 +240,23 @@ def test_sparse_page_table_allocator():
         sparse.reserve(1, None, 25)
     with pytest.raises(ValueError):
         PagedKVCache(8, 4, 2, 1, 4, 1, torch.float32, device="cpu", max_blocks_per_seq=9)
+
+
+def test_prefill_row_limit_survives_inference_mode():
+    """The reference's engine builds input_pos inside torch.inference_mode() (paged_inference.py:646-675,
+    1331); such tensors have no version counter.  The row limits are recomputed when a new step starts
+    (layer id not growing) or another positions tensor arrives."""
+    c = PagedKVCache(8, 4, 4, 2, 8, 1, torch.float32, device="cpu")
+    row_hi = torch.tensor([1, 5, 5, 5, 5, 6], dtype=torch.int32)
+    with torch.inference_mode():
+        bidx = torch.ones(1, 6, dtype=torch.int64)
+        m = A.HybridPrefillMask(c, bidx, torch.zeros(1, 6, dtype=torch.int64), 1, 2, 128, row_hi=row_hi)
+        pos = torch.arange(10, 16)[None]
+        with pytest.raises(RuntimeError):
+            pos._version  # what the key must not touch
+        lim0 = m.row_limit(pos, 0)
+        assert lim0.tolist() == [11, 15, 15, 15, 15, 16]
+        assert m.row_limit(pos, 1) is lim0  # later layers of the step reuse it
+        pos.add_(100)  # the engine's next step may reuse the buffer
+        assert m.row_limit(pos, 0).tolist() == [111, 115, 115, 115, 115, 116]
+        assert m.row_limit(torch.arange(6)[None], 1).tolist() == [1, 5, 5, 5, 5, 6]

@@ -114,3 +114,71 @@ def test_irregular_delimiters_keep_spans_contiguous():
             assert same.tolist() == list(range(same[0], same[-1] + 1))
             lo, hi = O.row_windows(bidx[None], ids[None], SOI, EOI)
             assert hi[q] == max(q + 1, same[-1] + 1)
+
+
+# ---------------------------------------------------------------- chunks that cut an image span
+
+@pytest.mark.parametrize("layout", LAYOUTS)
+def test_chunk_row_limits_equal_row_windows_on_whole_sequences(layout):
+    ids, bidx, pos, spans = packed_case(layout)
+    lo, hi = O.row_windows(bidx[None], ids[None], SOI, EOI)
+    got, status = O.chunk_row_limits(bidx[None], ids[None], SOI, EOI)
+    assert status == 0
+    real = bidx != 0
+    assert np.array_equal(got[real], hi[real])
+
+
+def test_chunk_row_limits_equal_row_windows_on_irregular_delimiters():
+    rng = np.random.default_rng(1)
+    clean = 0
+    for _ in range(600):
+        ids = rng.choice([SOI, EOI, IMG, TXT], size=16, p=[0.1, 0.1, 0.4, 0.4])
+        bidx = np.ones(16, dtype=np.int64)
+        got, status = O.chunk_row_limits(bidx[None], ids[None], SOI, EOI)
+        opened = np.cumsum(ids == SOI) - np.cumsum(ids == EOI)
+        assert bool(status & 1) == bool((opened < 0).any())
+        assert bool(status & 2) == bool(opened[-1] > 0)
+        if status == 0:
+            clean += 1
+            assert np.array_equal(got, O.row_windows(bidx[None], ids[None], SOI, EOI)[1])
+    assert clean > 20
+
+
+@pytest.mark.parametrize("segs", [
+    [("t", 3), ("i", 6), ("t", 5)],
+    [("i", 9), ("t", 4)],
+    [("t", 2), ("i", 3), ("t", 2), ("i", 5), ("t", 1)],
+])
+def test_chunk_boundaries_inside_the_image_span(segs):
+    """A sequence cut in two at every position: the second chunk's limits, with the span declared open
+    when the cut falls inside one, are the rows of the whole-sequence mask; the first chunk is refused
+    exactly when the cut falls inside a span (its rows would need keys that are not cached yet; a cut right
+    in front of the eoi counts as inside, since nothing in the first chunk says that the span ends there)."""
+    ids, bidx, pos, spans = packed_case([(3, segs)])
+    n = int((bidx != 0).sum())
+    ids, bidx = ids[:n], bidx[:n]
+    dense = O.hybrid_mask_dense(bidx[None], ids[None], SOI, EOI)
+    want = np.array([np.flatnonzero(dense[q])[-1] + 1 for q in range(n)])
+    for q in range(n):  # one limit per row is the whole mask: the allowed keys of a row are 0 .. want - 1
+        assert np.flatnonzero(dense[q]).tolist() == list(range(want[q]))
+    for p in range(1, n):
+        cut_inside = any(a < p <= e for a, e in spans)  # the soi lies before the cut, its eoi (index e) does not
+        head, status = O.chunk_row_limits(bidx[None, :p], ids[None, :p], SOI, EOI)
+        assert status == (2 if cut_inside else 0), p
+        if not cut_inside:
+            assert np.array_equal(head, want[:p])
+        tail, status = O.chunk_row_limits(bidx[None, p:], ids[None, p:], SOI, EOI, open_slots=[3] if cut_inside else [])
+        assert status == 0, p
+        assert np.array_equal(tail + p, want[p:]), p
+        if cut_inside:  # undeclared: the eoi closes nothing
+            assert O.chunk_row_limits(bidx[None, p:], ids[None, p:], SOI, EOI)[1] & 1
+
+
+def test_span_open_across_a_document_boundary_is_flagged():
+    ids = np.array([TXT, SOI, IMG, IMG, TXT, TXT, EOI, TXT])
+    bidx = np.array([1, 1, 1, 1, 2, 2, 2, 2])
+    # the reference's global counts would let rows 1..3 see rows 4..5 of the other document
+    dense = O.hybrid_mask_dense(bidx[None], ids[None], SOI, EOI)
+    assert dense[2, 5]
+    hi, status = O.chunk_row_limits(bidx[None], ids[None], SOI, EOI)
+    assert status == 3  # open at the boundary, and document 2's eoi closes nothing of its own
