@@ -364,7 +364,11 @@ __global__ __launch_bounds__(kThreads, (decode_waves_per_simd<E, D, G, kPerHeadK
   int64_t L = fp::load_index(a.input_pos, b, a.pos_i64) + 1;
   const int64_t trow = a.batch_idx[b];
   if (trow < 0 || trow >= a.max_batch) L = 0;
-  if (L > a.max_context) L = a.max_context;
+  // A position at or beyond max_context is outside what the launch was sized for: the context is read
+  // up to max_context from the pool, and the fresh row of a fused append is neither folded nor stored
+  // (it must not land on the slot of position max_context - 1, which holds a valid row).
+  const bool beyond = L > a.max_context;
+  if (beyond) L = a.max_context;
   auto lse_at = [&](int hq) -> float& {
     return a.lse[static_cast<int64_t>(b) * a.Hq + hq];
   };
@@ -383,7 +387,7 @@ __global__ __launch_bounds__(kThreads, (decode_waves_per_simd<E, D, G, kPerHeadK
   // Fused append: the newest token (position L - 1) is not in the pool yet.  The workgroup whose
   // range holds it reads that row from k_new / v_new, folds it in and writes it to its slot; the
   // pool is only read up to L - 2.
-  const bool owns_new = a.k_new != nullptr && L - 1 >= t0;  // t1 == L whenever L - 1 lies in this split
+  const bool owns_new = a.k_new != nullptr && !beyond && L - 1 >= t0;  // t1 == L whenever L - 1 lies in this split
   const int t1_pool = (owns_new && t1 == L) ? t1 - 1 : t1;
 
   // this lane's 16 bytes of the query row of every head of the group

@@ -215,6 +215,10 @@ def compiled_flex_attn_decode(q: Tensor, k: Tensor, v: Tensor, score_mod=None, b
     [1, Hc, n_slots, D].  `kernel_options` are Triton tuning knobs of the reference
     and are ignored.  `sinks` [Hq] float32 (not an argument of the reference's callable) applies
     the sink gate of `Attention._post_attention` (`model.py:122-126`) to the returned output.
+
+    The kernel attends positions 0 .. input_pos[b] of every sequence, i.e. the causal mask the engine
+    installs for a decode step (`q + input_pos[b] >= kv`, `paged_inference.py:797-801`); the `mask_mod` of
+    the logical mask is not evaluated, so a mask that hides earlier positions is outside this path.
     """
     if not isinstance(block_mask, PagedDecodeMask):
         if sinks is not None:
@@ -230,14 +234,17 @@ def compiled_flex_attn_decode(q: Tensor, k: Tensor, v: Tensor, score_mod=None, b
         raise RuntimeError("paged decode attention called before PagedKVCache.insert_kv for this step")
     if q.shape[2] != 1:
         raise RuntimeError("a PagedDecodeMask serves one query token per sequence")
+    if step.batch_idx.shape != block_mask.batch_idx.shape:
+        raise RuntimeError(
+            f"the mask was converted for {tuple(block_mask.batch_idx.shape)} sequences but the last insert_kv of this "
+            f"cache appended {tuple(step.batch_idx.shape)}: attention must follow the insert_kv of its own step")
     kv_rep = getattr(cache, "kv_rep", 1)
     wg_heads = k.shape[1] // kv_rep  # workgroups per sequence and split
+    workspace, split_tokens = cache.decode_launch(q.shape[0], q.shape[1], q.shape[3], block_mask.max_context, wg_heads)
     out, lse = ops.paged_decode(
         q, k[0], v[0], cache.page_table, block_mask.batch_idx, step.input_pos,
         cache.page_size, block_mask.max_context, scale=scale,
-        workspace=cache.decode_workspace(q.shape[0], q.shape[1], q.shape[3], block_mask.max_context, wg_heads),
-        split_tokens=cache.decode_split_tokens(q.shape[0], wg_heads, block_mask.max_context),
-        sinks=sinks, kv_rep=kv_rep,
+        workspace=workspace, split_tokens=split_tokens, sinks=sinks, kv_rep=kv_rep,
     )
     return _result(out, lse, return_aux, return_lse)
 

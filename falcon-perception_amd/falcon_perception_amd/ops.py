@@ -201,11 +201,15 @@ def paged_decode(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor, 
     batch_idx = batch_idx.contiguous()
     if scale is None:
         scale = 1.0 / math.sqrt(D)
+    if input_pos.numel() != B or batch_idx.numel() != B:
+        raise RuntimeError(f"input_pos ({input_pos.numel()}) and batch_idx ({batch_idx.numel()}) need one entry "
+                           f"per sequence of q ({B})")
     if split_tokens == 0:
         split_tokens = decode_split_tokens(B, Hc // kv_rep if kv_rep > 1 else Hc, max_context, page_size)
-    need = decode_workspace_bytes(B, Hq, D, max_context, split_tokens)
-    if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
-        workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+    if workspace is None:  # a workspace the caller brings is checked by the library against the launch
+        need = decode_workspace_bytes(B, Hq, D, max_context, split_tokens)
+        if need:
+            workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
     if out is None:
         out = torch.empty((B, Hq, 1, D), dtype=q.dtype, device=q.device)
     if lse is None:

@@ -85,6 +85,7 @@ class PagedKVCache(KVCacheBase):
         self.last_decode_step: StepMeta | None = None
         self.last_prefill_step: StepMeta | None = None
         self._workspace: Tensor | None = None
+        self._decode_launch: dict[tuple, tuple[int, int]] = {}
         self._prefill_workspace: Tensor | None = None
 
     # ------------------------------------------------------------------ append
@@ -316,14 +317,24 @@ class PagedKVCache(KVCacheBase):
         Sized on first use for the largest batch and the finest split any batch size
         can get, so its address never changes afterwards: HIP graphs captured for
         one batch bucket stay valid when another bucket runs."""
-        worst_b = max(B, self.max_batch_size)
-        finest = min(self.decode_split_tokens(1, Hc, max_context), self.decode_split_tokens(worst_b, Hc, max_context))
-        need = ops.decode_workspace_bytes(worst_b, Hq, D, max_context, finest)
-        if need == 0:
-            return None
-        if self._workspace is None or self._workspace.numel() < need:
-            self._workspace = torch.empty(need, dtype=torch.uint8, device=self.kv_cache.device)
-        return self._workspace
+        return self.decode_launch(B, Hq, D, max_context, Hc)[0]
+
+    def decode_launch(self, B: int, Hq: int, D: int, max_context: int, Hc: int) -> tuple[Tensor | None, int]:
+        """(workspace, split_tokens) of a decode launch of this shape.  The library is asked once per shape;
+        every later layer and step of the same batch bucket takes the answer from a dictionary, so an eager
+        decode step crosses into the library once per layer, for the launch itself."""
+        key = (B, Hq, D, max_context, Hc)
+        hit = self._decode_launch.get(key)
+        if hit is None:
+            worst_b = max(B, self.max_batch_size)
+            finest = min(self.decode_split_tokens(1, Hc, max_context),
+                         self.decode_split_tokens(worst_b, Hc, max_context))
+            need = ops.decode_workspace_bytes(worst_b, Hq, D, max_context, finest)
+            if need and (self._workspace is None or self._workspace.numel() < need):
+                self._workspace = torch.empty(need, dtype=torch.uint8, device=self.kv_cache.device)
+            hit = (need, self.decode_split_tokens(B, Hc, max_context))
+            self._decode_launch[key] = hit
+        return (self._workspace if hit[0] else None), hit[1]
 
     def prefill_workspace(self, Lq: int, Hq: int, D: int, Hc: int, dtype: torch.dtype):
         """Scratch with which the prefill kernel cuts a small launch along the keys as well, owned by the

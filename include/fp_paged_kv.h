@@ -232,6 +232,9 @@ int fp_paged_decode_merge(const void* q, int64_t q_stride_b, int64_t q_stride_h,
  * k_new / v_new, folds it into the attention and writes it to its pool slot.
  *
  *   k_new, v_new  [B, Hc, 1, D], element strides (b, h); pool_k / pool_v are written
+ * A sequence with input_pos >= max_context lies outside what the launch was sized for: its fresh row
+ * is neither stored nor attended, the pool stays as it was, and the result covers positions
+ * 0 .. max_context - 1 as fp_paged_decode would return it.
  * All other arguments as fp_paged_decode.
  */
 int fp_paged_decode_append(const void* k_new, const void* v_new,

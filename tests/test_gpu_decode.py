@@ -354,3 +354,43 @@ def test_no_pass_writes_outside_the_workspace_it_asked_for(B, ctx):
     assert bool((buf[need:] == 0x5A).all())
     eo, el = oracle_decode(st, q, pos)
     assert_close(out, lse, eo, el, dtype)
+
+
+@pytest.mark.parametrize("split,B", [(64, 3), (0, 3), (64, 80)])
+def test_fused_append_beyond_max_context_leaves_the_pool_alone(split, B):
+    """A sequence whose new position is max_context or more lies outside what the launch was sized for: its
+    fresh row is neither stored (the slot of position max_context - 1 holds a valid row) nor attended; the
+    other sequences of the step append as usual.  Also on the evenly cut launch (B = 80)."""
+    dtype, P, Hc, G, D, ctx = torch.bfloat16, 16, 2, 2, 128, 256
+    st = PagedState(41, n_pages=B * 18 + 4, page_size=P, max_batch=B + 2, Hc=Hc, D=D, dtype=dtype)
+    lens = [ctx, ctx + 5, 100] + [37 + i for i in range(B - 3)]  # tokens cached before the step
+    for L in lens:
+        st.add_sequence(L + 1)
+    st.lens = lens
+    st.prefill_random()
+    before = st.cache.kv_cache.clone()
+    q = randn(st.gen, (B, Hc * G, 1, D), dtype)
+    k_new = randn(st.gen, (B, Hc, 1, D), dtype)
+    v_new = randn(st.gen, (B, Hc, 1, D), dtype)
+    pos = torch.tensor(lens, dtype=torch.int32)
+    out, lse = run_decode(st, q, pos, k_new=k_new.to(DEV), v_new=v_new.to(DEV), split_tokens=split, max_context=ctx)
+    # expected pool: the rows of sequences 2.. appended by the oracle's decode append, 0 and 1 untouched
+    ref = before.double().cpu().numpy()
+    O.append_decode(ref, 0, f64(k_new[2:]), f64(v_new[2:]), st.mirror.page_table, np.array(st.slots[2:]),
+                    np.array(lens[2:])[:, None], P)
+    assert np.array_equal(st.cache.kv_cache.double().cpu().numpy(), ref)
+    # expected attention: positions 0 .. ctx - 1 for the two sequences beyond, the full context for the rest
+    seen = pos.clone()
+    seen[:2] = ctx - 1
+    eo, el = oracle_decode(st, q, seen)
+    assert_close(out, lse, eo, el, dtype)
+
+
+def test_one_position_and_slot_per_sequence_is_required():
+    st = PagedState(42, n_pages=8, page_size=16, max_batch=6, Hc=1, D=64, dtype=torch.bfloat16)
+    for L in (5, 9, 20):
+        st.add_sequence(L)
+    st.prefill_random()
+    q = randn(st.gen, (3, 1, 1, 64), torch.bfloat16)
+    with pytest.raises(RuntimeError, match="one entry per sequence"):
+        run_decode(st, q, torch.tensor([4, 8], dtype=torch.int32))
