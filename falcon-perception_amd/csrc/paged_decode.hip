@@ -23,6 +23,8 @@
 //           (through the workspace, by the merge kernel) are combined at the end.
 #include "fp_common.h"
 
+#include <atomic>
+
 #include <hip/hip_bf16.h>
 #include <hip/hip_fp16.h>
 #include <math.h>
@@ -1087,3 +1089,74 @@ extern "C" int fp_paged_decode_append(const void* k_new, const void* v_new, int6
   return decode_entry(kPhasePartial | kPhaseMerge, &fresh, FP_DECODE_ARGS);
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// fp_paged_decode for callers that cannot allocate: the split-K partial results go to an array that
+// lives in the library's device image instead of a caller-owned workspace.
+//
+// `scratch` below is, in host code, only a handle of the device symbol: its device address differs
+// per GPU and is asked for once per device with hipGetSymbolAddress, on the entry point's first call
+// on that device (with that device current).  Only that address is ever handed to a kernel.  Every
+// launch on a GPU shares the GPU's one array: calls that overlap on one GPU (two streams, two
+// threads) race on it.  The partial pass writes every row the merge pass reads, so the contents left
+// by an earlier call never need clearing.
+constexpr int64_t kScratchBytes = FP_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// device address of `scratch` on the current device, nullptr + error message on failure
+void* scratch_address() {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    fp::fail(FP_ERR_LAUNCH, "fp_paged_decode_noalloc: hipGetDevice: %s (device %d)", hipGetErrorString(e), dev);
+    return nullptr;
+  }
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p) return p;
+  e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+  if (e != hipSuccess || !p) {
+    (void)hipGetLastError();
+    fp::fail(FP_ERR_LAUNCH, "fp_paged_decode_noalloc: hipGetSymbolAddress(scratch) on device %d: %s", dev,
+             hipGetErrorString(e));
+    return nullptr;
+  }
+  g_scratch_ptr[dev].store(p, std::memory_order_release);  // two first calls racing store the same address
+  return p;
+}
+}  // namespace
+
+extern "C" int fp_paged_decode_noalloc(const void* q, int64_t q_stride_b, int64_t q_stride_h, const void* pool_k,
+                                       const void* pool_v, const int64_t* page_table, int64_t pt_row_stride,
+                                       const int64_t* batch_idx, const void* input_pos, int pos_index_type,
+                                       void* out, int64_t out_stride_b, int64_t out_stride_h, float* lse,
+                                       const float* sinks, int32_t B, int32_t Hq, int32_t Hc, int32_t kv_rep,
+                                       int32_t D, int32_t page_size, int32_t n_pages, int32_t max_batch,
+                                       int64_t n_slots, int32_t max_context, int32_t split_tokens, float scale,
+                                       int dtype, void* stream) {
+  // size the partial results exactly as decode_entry will, and refuse what the array cannot hold
+  if (B < 0 || Hq <= 0 || Hc <= 0 || D <= 0 || page_size <= 0 || max_context < 0 || split_tokens < 0 || kv_rep < 1)
+    return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode_noalloc: bad dimension");
+  int st = split_tokens;
+  if (st == 0) st = default_split_tokens(B, kv_rep > 1 ? Hq / kv_rep : Hc, max_context, page_size);
+  if (st % 64) return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode_noalloc: split_tokens must be a multiple of 64");
+  const int64_t ns = n_splits_for(max_context, st);
+  const int64_t need = ns > 1 ? static_cast<int64_t>(B) * Hq * ns * (D + 2) * static_cast<int64_t>(sizeof(float)) : 0;
+  if (need > kScratchBytes)
+    return fp::fail(FP_ERR_WORKSPACE,
+                    "fp_paged_decode_noalloc: this launch needs %lld bytes of split-K partial results, the library's "
+                    "array holds %lld; use fp_paged_decode with a caller-owned workspace, or a larger split_tokens",
+                    static_cast<long long>(need), static_cast<long long>(kScratchBytes));
+  void* ws = nullptr;
+  if (need) {
+    ws = scratch_address();
+    if (!ws) return FP_ERR_LAUNCH;
+  }
+  return decode_entry(kPhasePartial | kPhaseMerge, nullptr, q, q_stride_b, q_stride_h, pool_k, pool_v, page_table,
+                      pt_row_stride, batch_idx, input_pos, pos_index_type, out, out_stride_b, out_stride_h, lse, sinks,
+                      ws, need ? kScratchBytes : 0, B, Hq, Hc, kv_rep, D, page_size, n_pages, max_batch, n_slots,
+                      max_context, st, scale, dtype, stream);
+}

@@ -242,6 +242,40 @@ def paged_decode(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor, 
     return out, lse
 
 
+def paged_decode_noalloc(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor, batch_idx: Tensor,
+                         input_pos: Tensor, page_size: int, max_context: int, out: Tensor, lse: Tensor, *,
+                         scale: float | None = None, split_tokens: int = 0, sinks: Tensor | None = None,
+                         kv_rep: int = 1) -> tuple[Tensor, Tensor]:
+    """`paged_decode` for callers that may not allocate: the caller brings `out` [B, Hq, 1, D] and `lse`
+    [B, Hq, 1], the split-K partial results go to an array inside the library (`_native.NOALLOC_SCRATCH_BYTES`;
+    a larger launch raises), and neither this wrapper nor the library allocates.  Calls that overlap on one
+    GPU share that array and race."""
+    N.require_cuda(q, pool_k, pool_v, page_table, batch_idx, input_pos, out, lse)
+    B, Hq, Sq, D = q.shape
+    Hc, n_slots, Dp = pool_k.shape
+    if Sq != 1 or Dp != D or pool_v.shape != pool_k.shape or pool_k.dtype != q.dtype or pool_v.dtype != q.dtype:
+        raise RuntimeError("q / pool shape or dtype mismatch")
+    if q.stride(3) != 1 or not input_pos.is_contiguous() or not batch_idx.is_contiguous():
+        raise RuntimeError("q rows, input_pos and batch_idx must be dense (nothing is copied here)")
+    if input_pos.numel() != B or batch_idx.numel() != B:
+        raise RuntimeError("input_pos and batch_idx need one entry per sequence of q")
+    if out.shape != (B, Hq, 1, D) or out.dtype != q.dtype or out.stride(3) != 1:
+        raise RuntimeError("out must be [B, Hq, 1, D] of the q dtype with dense rows")
+    if lse.shape != (B, Hq, 1) or lse.dtype != torch.float32 or not lse.is_contiguous():
+        raise RuntimeError("lse must be contiguous float32 [B, Hq, 1]")
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    rc = N.lib().fp_paged_decode_noalloc(
+        q.data_ptr(), q.stride(0), q.stride(1), pool_k.data_ptr(), pool_v.data_ptr(),
+        page_table.data_ptr(), page_table.stride(0), batch_idx.data_ptr(),
+        input_pos.data_ptr(), N.index_code(input_pos),
+        out.data_ptr(), out.stride(0), out.stride(1), lse.data_ptr(), _sinks_ptr(sinks, Hq, q.device),
+        B, Hq, Hc, kv_rep, D, page_size, page_table.shape[1], page_table.shape[0],
+        n_slots, max_context, split_tokens, scale, N.dtype_code(q.dtype), N.stream_ptr(q.device))
+    N.check(rc, "fp_paged_decode_noalloc")
+    return out, lse
+
+
 def hybrid_row_limits(input_ids: Tensor, soi_id: int, eoi_id: int, batch_idx: Tensor | None = None,
                       open_at_start: Tensor | None = None, status: Tensor | None = None) -> Tensor:
     """Packed index one past the last key each packed row may see: max(q + 1, end of q's image span).

@@ -255,6 +255,33 @@ int fp_paged_decode_append(const void* k_new, const void* v_new,
                            void* stream);
 
 /*
+ * fp_paged_decode without a workspace argument, for callers that cannot allocate device memory:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart
+ * in the reference.  The split-K partial results go to an array of FP_NOALLOC_SCRATCH_BYTES that is
+ * part of the library's device image (every GPU the library runs on holds its own copy until the
+ * process ends); the call allocates and frees nothing.  The first call on a device looks the array's
+ * address up once (hipGetSymbolAddress, with that device current).
+ *  - A launch whose partial results (fp_paged_decode_workspace_bytes for the same shape) exceed
+ *    FP_NOALLOC_SCRATCH_BYTES is refused with FP_ERR_WORKSPACE.
+ *  - All calls on one GPU share that GPU's array: calls that overlap there (different streams or
+ *    threads) race.  Nothing needs clearing between calls.
+ * Arguments and results as fp_paged_decode.
+ */
+#define FP_NOALLOC_SCRATCH_BYTES (64ll << 20)
+int fp_paged_decode_noalloc(const void* q, int64_t q_stride_b, int64_t q_stride_h,
+                            const void* pool_k, const void* pool_v,
+                            const int64_t* page_table, int64_t pt_row_stride,
+                            const int64_t* batch_idx,
+                            const void* input_pos, int pos_index_type,
+                            void* out, int64_t out_stride_b, int64_t out_stride_h,
+                            float* lse, const float* sinks,
+                            int32_t B, int32_t Hq, int32_t Hc, int32_t kv_rep, int32_t D,
+                            int32_t page_size, int32_t n_pages, int32_t max_batch,
+                            int64_t n_slots, int32_t max_context, int32_t split_tokens,
+                            float scale, int dtype,
+                            void* stream);
+
+/*
  * Tail of Attention._pre_attention (model.py:110-119) and the cache insert that follows it
  * (model.py:150-153 -> PagedKVCache.assign / assign_prefill_no_paging, paged_attention.py:184-232,
  * 364-393) in one pass: RMS norm of q and k over head_dim (no weight), repeat of k and v to the
