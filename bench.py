@@ -18,6 +18,7 @@ import argparse
 import json
 import math
 import os
+import statistics
 import sys
 import time
 from dataclasses import dataclass, field
@@ -44,12 +45,26 @@ DECODE_WORKLOADS = {
                    kv_rep=2),
     "cfg4d": dict(seed=4, dtype="bf16", B=32, Hq=16, Hc=8, D=128, P=64, n_pages=8192, prefix=0, lo=512, hi=8192),
     "cfg5": dict(seed=5, dtype="bf16", B=256, Hq=32, Hc=8, D=128, P=128, n_pages=None, prefix=4096, lo=256, hi=12288),
+    # cfg2 at the head_dim of the reference's OCR and 300M variants (reference __init__.py:78-85)
+    "cfg2d64": dict(seed=2, dtype="bf16", B=64, Hq=16, Hc=8, D=64, P=128, n_pages=4096, prefix=1024, lo=64, hi=3072),
 }
 DTYPES = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
 
-# HBM bytes per launch of paged_decode_kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
-# (profiles/), scaled by the same counters on a plain copy of known size; None = not measured
-TRAFFIC_BYTES = {"cfg2": 671.4e6}  # profiles/paged_decode_cfg2_hbm_traffic.md
+
+
+def profiled_traffic(kernel: str, workload: str) -> float | None:
+    """HBM bytes per launch of `kernel` at `workload` as a rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE pair
+    measured them (each scaled by the same counter on a plain copy of known size): the line
+    `traffic_bytes_per_launch = N` of profiles/<kernel>_<workload>_hbm_traffic.md, None when no such
+    summary has been recorded."""
+    import re
+
+    path = os.path.join(ROOT, "profiles", f"{kernel}_{workload}_hbm_traffic.md")
+    try:
+        m = re.search(r"traffic_bytes_per_launch\s*=\s*([0-9.eE+]+)", open(path).read())
+    except OSError:
+        return None
+    return float(m.group(1)) if m else None
 
 
 @dataclass
@@ -209,6 +224,10 @@ PREFILL_WORKLOADS = {
     "cfg3one": dict(seed=3, dtype="bf16", n_seq=1, Hq=16, Hc=8, D=128, P=128, prefix_lo=4096, prefix_hi=4096, chunk=512),
     # cfg3 in the reference's default dtype (reference server/config.py:38)
     "cfg3f32": dict(seed=3, dtype="f32", n_seq=8, Hq=16, Hc=8, D=128, P=128, prefix_lo=256, prefix_hi=4096, chunk=512),
+    # cfg3 on the cache the reference's engine builds: one cached head per query head (paged_inference.py:321-330)
+    "cfg3x": dict(seed=3, dtype="bf16", n_seq=8, Hq=16, Hc=16, D=128, P=128, prefix_lo=256, prefix_hi=4096, chunk=512),
+    # cfg3 at the head_dim of the OCR and 300M variants
+    "cfg3d64": dict(seed=3, dtype="bf16", n_seq=8, Hq=16, Hc=8, D=64, P=128, prefix_lo=256, prefix_hi=4096, chunk=512),
 }
 
 
@@ -312,17 +331,22 @@ def make_prefill_case(name: str, device="cuda") -> PrefillCase:
 # timing
 # --------------------------------------------------------------------------
 
-def time_steps(fn, steps: int, warmup: int) -> float:
-    """Wall-clock ms per step of `fn`, launches back to back, synchronised on both sides."""
+def time_steps(fn, steps: int, warmup: int, samples: int = 21) -> float:
+    """Wall-clock ms per step of `fn`: a sample is exactly `steps` launches back to back, synchronised on
+    both sides; the median of `samples` such regions is returned (after a clock warm-up and `warmup`
+    untimed steps)."""
     warm_clocks(fn)
     for _ in range(warmup):
         fn()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        fn()
-    torch.cuda.synchronize()
-    return (time.perf_counter() - t0) * 1e3 / steps
+    regions = []
+    for _ in range(samples):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        regions.append((time.perf_counter() - t0) * 1e3 / steps)
+    return statistics.median(regions)
 
 
 def warm_clocks(fn, seconds: float = 0.2) -> None:
@@ -337,17 +361,19 @@ def warm_clocks(fn, seconds: float = 0.2) -> None:
 
 
 def event_ms(fn, steps: int) -> float:
-    """Average device ms per call of `fn`, HIP events on the stream the kernels run on."""
+    """Device ms per call of `fn`: HIP events on the stream the kernels run on around every call, median of
+    at least 20 calls."""
     warm_clocks(fn)
+    n = max(steps, 20)
     stream = torch.cuda.current_stream()
-    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    for i in range(steps):
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+    for i in range(n):
         starts[i].record(stream)
         fn()
         ends[i].record(stream)
     torch.cuda.synchronize()
-    return sum(s.elapsed_time(e) for s, e in zip(starts, ends)) / steps
+    return statistics.median(s.elapsed_time(e) for s, e in zip(starts, ends))
 
 
 def graph_ms(fn, steps: int) -> float:
@@ -363,11 +389,15 @@ def graph_ms(fn, steps: int) -> float:
     g.replay()
     torch.cuda.synchronize()
     warm_clocks(g.replay)
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        g.replay()
-    torch.cuda.synchronize()
-    return (time.perf_counter() - t0) * 1e3 / steps
+    regions = []
+    for _ in range(11):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            g.replay()
+        torch.cuda.synchronize()
+        regions.append((time.perf_counter() - t0) * 1e3 / steps)
+    return statistics.median(regions)
 
 
 def model_depth_graph_ms(case: "DecodeCase", steps: int, layers: int = MODEL_LAYERS) -> float | None:
@@ -529,6 +559,8 @@ def prefill_rate(steps: int = 10, name: str = "cfg3") -> dict:
             "cfg3w": "cfg3w: the same 8 sequences prefilled whole (prefix + chunk rows in one step, prefix rows see "
                      "their whole image span), 16 q / 8 kv heads, D 128",
             "cfg3f32": "cfg3 in fp32",
+            "cfg3x": "cfg3 on the reference engine's cache: one cached head per query head (16 q / 16 cached heads)",
+            "cfg3d64": "cfg3 at head_dim 64 (the reference's OCR and 300M variants)",
             "cfg3one": "one sequence alone: paged prefix 4096, 512-token chunk, 16 q / 8 kv heads, D 128 "
                        "(cut along the keys into 8 shares + merge pass)"}[name]
     res = {"workload": what, "query_rows": int(case.q.shape[2]), "paged_prefill_ms": ms, "tflops": tf,
@@ -557,7 +589,140 @@ def small_batch_decode(steps: int = 200) -> dict:
     return out
 
 
-def cpu_baseline(case: DecodeCase, budget_s: float = 20.0) -> dict:
+def decode_leg(name: str, steps: int = 20, hbm_budget_gb: float | None = None, cpu: bool = False) -> dict:
+    """One more decode workload next to the headline: the fused step (append inside the split-K pass + merge)
+    timed like the headline, the split-K pass alone by events, both priced with the workload's algorithmic
+    bytes."""
+    if name == "cfg5" and hbm_budget_gb is None:
+        free, _ = torch.cuda.mem_get_info()
+        hbm_budget_gb = min(180.0, (free - 24e9) / 1e9)
+        if hbm_budget_gb < 30:
+            return {"skipped": f"only {free / 1e9:.0f} GB of HBM free: no room for a long-context pool"}
+    case = make_decode_case(name, hbm_budget_gb=hbm_budget_gb)
+    c = case.cfg
+    ms_step = time_steps(case.run_fused, steps, 5, samples=11)
+    ms_partial = event_ms(lambda: case.attend("partial"), steps)
+    alg_decode, alg_append = case.bytes_decode(), case.bytes_append()
+    gbps = (alg_decode + alg_append) / (ms_step * 1e-3) / 1e9
+    kernel_gbps = alg_decode / (ms_partial * 1e-3) / 1e9
+    res = {
+        "workload": f"batch {c['B']}, {c['Hq']} q / {c['Hc']} cached heads"
+                    + (f" (V read once per {c['kv_rep']} heads)" if c.get("kv_rep", 1) > 1 else "")
+                    + f", head_dim {c['D']}, {c['dtype']}, page_size {c['P']}, {c['n_pages']}-page pool "
+                    f"({case.cache.kv_cache.numel() * case.cache.kv_cache.element_size() / 1e9:.1f} GB), contexts "
+                    f"{c['prefix']}+U[{c['lo']},{c['hi']}]",
+        "ms_per_step": ms_step, "gbps": gbps, "pct_of_hbm_peak": 100.0 * gbps / HBM_PEAK_GBPS,
+        "decode_tok_s_per_layer": c["B"] / (ms_step * 1e-3), "algorithmic_bytes": alg_decode + alg_append,
+        "roofline": {"bound": "hbm", "kernel": "paged_decode_kernel", "achieved": kernel_gbps, "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": kernel_gbps / HBM_PEAK_GBPS, "ms": ms_partial,
+                     "traffic": profiled_traffic("paged_decode", name), "algorithmic_bytes": alg_decode},
+    }
+    if cpu:
+        res["cpu_baseline"] = cpu_baseline(case, budget_s=5.0, min_reps=20)
+        res["gpu_over_cpu"] = gbps / res["cpu_baseline"]["value"]
+    del case
+    torch.cuda.empty_cache()
+    return res
+
+
+def cfg4_mixed_step(steps: int = 6) -> dict:
+    """BASELINE configs[3] as one mixed step: the fused decode step of the running sequences (contexts
+    U[512, 8192]) plus the append and chunked-prefill attention of 4 chunks of 1024 tokens (2 fresh sequences
+    whose first 512 tokens are an image span, 2 continuing after a 2048-token paged prefix), page size 64,
+    16 q / 8 kv heads, D 128, bf16, 8192-page pool.  Between steps the chunk sequences leave and a quarter of
+    the decode sequences is erased and replaced through the allocator, so the page tables stay fragmented;
+    that host-side churn (and the prefill of the newcomers' contexts) lies outside the timed region."""
+    from falcon_perception_amd import ops
+    from falcon_perception_amd.paged_attention import PagedKVCache
+
+    dev, dtype = "cuda", torch.bfloat16
+    P, Hq, Hc, D, n_pages = 64, 16, 8, 128, 8192
+    gen = torch.Generator().manual_seed(4)
+    dgen = torch.Generator(device=dev).manual_seed(4)
+    cache = PagedKVCache(n_pages, P, 64, Hc, D, 1, dtype, device=dev)
+    cache.free_pages = (torch.randperm(n_pages - 1, generator=gen) + 1).tolist()
+    cache.kv_cache.view(-1).normal_(generator=dgen)
+    pk, pv = cache.kv_cache[0, 0, 0], cache.kv_cache[0, 1, 0]
+    rnd = lambda *shape: torch.randn(shape, generator=dgen, device=dev, dtype=torch.float32).to(dtype)
+
+    def admit(length):
+        b = cache.allocate()
+        cache.reserve(b, torch.tensor([b], device=dev), length)
+        return b
+
+    ctx = {}
+    for L in torch.randint(512, 8193, (32,), generator=gen).tolist():
+        if cache.can_reserve(L + 64):
+            ctx[admit(L + 64)] = L  # the pool already holds N(0,1) rows everywhere
+    max_context = 8192 + 64
+    samples, work = [], []
+    q4, k4, v4 = rnd(1, Hq, 4096, D), rnd(1, Hc, 4096, D), rnd(1, Hc, 4096, D)
+    for step in range(steps + 2):
+        chunks = []
+        for kind in ("fresh", "fresh", "cont", "cont"):
+            if kind == "fresh":
+                chunks.append((admit(1024), 0, [max(t + 1, 512) for t in range(1024)]))
+            else:
+                chunks.append((admit(2048 + 1024), 2048, [2048 + t + 1 for t in range(1024)]))
+        bidx = torch.cat([torch.full((1024,), s, dtype=torch.int64) for s, _, _ in chunks])[None].to(dev)
+        pos = torch.cat([torch.arange(st, st + 1024, dtype=torch.int64) for _, st, _ in chunks])[None].to(dev)
+        lims = [x for _, _, l in chunks for x in l]
+        lim = torch.tensor(lims, dtype=torch.int32, device=dev)
+        slots = sorted(ctx)
+        B = len(slots)
+        bt = torch.tensor(slots, dtype=torch.int64, device=dev)
+        pt = torch.tensor([ctx[s] for s in slots], dtype=torch.int32, device=dev)
+        k1, v1, q1 = rnd(B, Hc, 1, D), rnd(B, Hc, 1, D), rnd(B, Hq, 1, D)
+        split = ops.decode_split_tokens(B, Hc, max_context, P)
+        ws = torch.empty(max(ops.decode_workspace_bytes(B, Hq, D, max_context, split), 16), dtype=torch.uint8, device=dev)
+        pws = cache.prefill_workspace(4096, Hq, D, Hc, dtype)
+        out1 = torch.empty_like(q1)
+        lse1 = torch.empty((B, Hq, 1), dtype=torch.float32, device=dev)
+        out4 = torch.empty_like(q4)
+        lse4 = torch.empty((1, Hq, 4096), dtype=torch.float32, device=dev)
+
+        def mixed():
+            ops.paged_decode(q1, pk, pv, cache.page_table, bt, pt, P, max_context, split_tokens=split, workspace=ws,
+                             out=out1, lse=lse1, k_new=k1, v_new=v1)
+            cache.insert_kv(0, k4, v4, input_pos=pos, batch_idx=bidx)
+            ops.paged_prefill(q4, pk, pv, cache.page_table, bidx, lim, P, out=out4, lse=lse4, workspace=pws)
+
+        if step == 0:
+            warm_clocks(mixed)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        mixed()
+        e1.record()
+        torch.cuda.synchronize()
+        e = 2
+        dec_bytes = (sum(ctx[s] + 1 for s in slots) * 2 * Hc * D * e + 2 * B * Hq * D * e + 4 * B * Hq
+                     + 8 * sum(math.ceil((ctx[s] + 1) / P) for s in slots) + 2 * B * 2 * Hc * D * e + 8 * B)
+        app_bytes = 2 * 4096 * 2 * Hc * D * e + 8 * 4096
+        flops = 4 * D * Hq * sum(lims)
+        if step >= 2:  # the first two steps are warm-up
+            samples.append(e0.elapsed_time(e1))
+            work.append((B, dec_bytes, app_bytes, flops))
+        for s in slots:
+            ctx[s] += 1
+        for s, _, _ in chunks:
+            cache.erase(s)
+        leaving = [slots[i] for i in torch.randperm(B, generator=gen)[: B // 4].tolist()]
+        for s in leaving:
+            cache.erase(s)
+            del ctx[s]
+        for L in torch.randint(512, 8193, (len(leaving),), generator=gen).tolist():
+            if cache.can_reserve(L + 64):
+                ctx[admit(L + 64)] = L
+    ms = statistics.median(samples)
+    B, dec_bytes, app_bytes, flops = work[samples.index(ms)] if ms in samples else work[-1]
+    return {"workload": "cfg4: fused decode step of the running sequences + append and chunked-prefill attention of "
+                        "4 x 1024-token chunks, one quarter of the decode sequences replaced between steps",
+            "steps_timed": len(samples), "ms_per_mixed_step": ms, "decode_sequences": B,
+            "decode_bytes": dec_bytes, "chunk_append_bytes": app_bytes, "prefill_flops": flops,
+            "ms_samples": samples}
+
+
+def cpu_baseline(case: DecodeCase, budget_s: float = 20.0, min_reps: int = 3) -> dict:
     """The reference's op sequence for one decode layer-step, ported to torch-CPU, timed on the
     host cores on a batch subset sized to roughly `budget_s` seconds."""
     from oracle import cpu_path
@@ -582,39 +747,56 @@ def cpu_baseline(case: DecodeCase, budget_s: float = 20.0) -> dict:
     probe = time.perf_counter() - t0
     per_seq = probe / n
     nb = int(max(1, min(c["B"], (budget_s / 3) / max(per_seq, 1e-6))))
-    reps, total = 0, 0.0
-    while reps < 3 and total < budget_s:
+    times, total = [], 0.0
+    while len(times) < min_reps or (len(times) < 20 and total < budget_s):
         t0 = time.perf_counter()
         one(nb)
-        total += time.perf_counter() - t0
-        reps += 1
-    sec = total / reps
+        times.append(time.perf_counter() - t0)
+        total += times[-1]
+        if total > 1.5 * budget_s:
+            break
+    reps, sec = len(times), statistics.median(times)
     ctx = [L + 1 for L in case.lens[:nb]]
     e = case.q.element_size()
     alg = (sum(ctx) * 2 * c["Hc"] * c["D"] * e + 2 * nb * c["Hq"] * c["D"] * e + 4 * nb * c["Hq"]
            + 8 * sum(math.ceil(x / c["P"]) for x in ctx) + 2 * nb * 2 * c["Hc"] * c["D"] * e + 8 * nb)
     return {
         "value": alg / sec / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
-        "sample": f"{nb} of {c['B']} sequences of {case.name}, {reps} repetitions, one layer-step each "
+        "sample": f"{nb} of {c['B']} sequences of {case.name}, median of {reps} repetitions, one layer-step each "
                   f"(append + block-id gather + dense masked attention over the whole pool, fp32)",
         "decode_tok_s_per_layer": nb / sec, "ms_per_step_sample": sec * 1e3,
     }
 
 
+def calibration_copies() -> None:
+    """Five launches of a plain elementwise copy of known traffic (1 GiB read, 1 GiB written), so that a
+    rocprofv3 --pmc run of this process holds the scale of each counter next to the kernels of interest."""
+    src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")
+    dst = torch.empty_like(src)
+    for _ in range(5):
+        torch.mul(src, 2.0, out=dst)
+    torch.cuda.synchronize()
+    del src, dst
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="cfg2", choices=sorted(DECODE_WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--decode-only", action="store_true", help="skip the append/gather/prefill side measurements")
+    ap.add_argument("--decode-only", action="store_true",
+                    help="only the headline workload: no other configs, no append/gather/prefill measurements")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run a plain 1 GiB elementwise copy (x * 2) a few times, so a rocprofv3 --pmc run of this "
-                         "command holds a kernel of known traffic next to the decode kernel")
-    ap.add_argument("--hbm-budget-gb", type=float, default=None, help="pool size for cfg5")
+                         "command holds a kernel of known traffic next to the kernels of interest")
+    ap.add_argument("--hbm-budget-gb", type=float, default=None, help="pool size for cfg5 (default: what fits, at most 180)")
     ap.add_argument("--prefill-only", default=None, choices=sorted(PREFILL_WORKLOADS),
                     help="time only the chunked-prefill attention of this workload and print its JSON (for profiling)")
+    ap.add_argument("--pieces-only", action="store_true",
+                    help="time only KV append, page gather and the fused norm + rotary append at 32768 tokens and print "
+                         "their JSON (for profiling)")
     args = ap.parse_args()
 
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -628,23 +810,20 @@ def main() -> int:
     from falcon_perception_amd import _native
 
     _native.lib()  # fail loudly if the HIP library is not built
+    if args.pmc_calibration:
+        calibration_copies()
     if args.prefill_only:
         print(json.dumps(prefill_rate(max(args.steps, 1), args.prefill_only)))
+        return 0
+    if args.pieces_only:
+        print(json.dumps(append_gather_rates(max(args.steps, 1))))
         return 0
     case = make_decode_case(args.workload, hbm_budget_gb=args.hbm_budget_gb)
     c = case.cfg
 
-    if args.pmc_calibration:
-        src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")  # 1 GiB read + 1 GiB written per copy
-        dst = torch.empty_like(src)
-        for _ in range(5):
-            torch.mul(src, 2.0, out=dst)  # an elementwise kernel of its own name: reads 1 GiB, writes 1 GiB
-        torch.cuda.synchronize()
-        del src, dst
-
     ms_step = time_steps(case.run_fused, args.steps, args.warmup)
-    ms_separate = time_steps(case.run, args.steps, args.warmup)
-    ms_gated = time_steps(case.run_fused_gated, args.steps, args.warmup)
+    ms_separate = time_steps(case.run, args.steps, args.warmup, samples=5)
+    ms_gated = time_steps(case.run_fused_gated, args.steps, args.warmup, samples=5)
     ms_graph = graph_ms(case.run_fused, args.steps)
     ms_decode = event_ms(case.attend, args.steps)
     ms_partial = event_ms(lambda: case.attend("partial"), args.steps)  # the dominant kernel alone
@@ -667,6 +846,8 @@ def main() -> int:
                                f"head_dim {c['D']}, page_size {c['P']}, {c['n_pages']}-page pool, contexts "
                                f"{c['prefix']}+U[{c['lo']},{c['hi']}], seed {c['seed']}",
                    "tokens_in_cache": sum(case.lens), "split_tokens": case.split_tokens},
+        "timing": "ms_per_step = median of 21 regions of exactly `steps` back-to-back steps, synchronised on both "
+                  "sides; kernel times = median of >= 20 HIP-event samples on the launch stream",
         "pct_of_hbm_peak": 100.0 * value / HBM_PEAK_GBPS,
         "decode_tok_s_per_layer": c["B"] / (ms_step * 1e-3),
         "decode_tok_s_model": c["B"] / (ms_step * 1e-3) / MODEL_LAYERS,
@@ -685,21 +866,33 @@ def main() -> int:
                     "kv_append_ms": ms_append, "kv_append_gbps": alg_append / (ms_append * 1e-3) / 1e9},
         "roofline": {"bound": "hbm", "kernel": "paged_decode_kernel", "achieved": achieved,
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
-                     "traffic": TRAFFIC_BYTES.get(case.name), "algorithmic_bytes": alg_decode},
+                     "traffic": profiled_traffic("paged_decode", case.name), "algorithmic_bytes": alg_decode},
     }
-    if not args.decode_only:
-        result["prefill_sized"] = append_gather_rates()
-        result["chunked_prefill"] = prefill_rate()
-        result["chunked_prefill_fp32"] = prefill_rate(name="cfg3f32")
-        result["chunked_prefill_one_sequence"] = prefill_rate(name="cfg3one")
-        result["decode_small_batch"] = small_batch_decode()
-        ms_model = model_depth_graph_ms(case, args.steps)  # last: it takes and returns 56 GiB
-        if ms_model is not None:
-            result["ms_all_layers_hip_graph"] = ms_model
-            result["decode_tok_s_model_measured"] = c["B"] / (ms_model * 1e-3)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(case)
         result["gpu_over_cpu"] = value / result["cpu_baseline"]["value"]
+    if not args.decode_only:
+        ms_model = model_depth_graph_ms(case, args.steps)  # takes and returns 56 GiB
+        if ms_model is not None:
+            result["ms_all_layers_hip_graph"] = ms_model
+            result["decode_tok_s_model_measured"] = c["B"] / (ms_model * 1e-3)
+        del case
+        torch.cuda.empty_cache()
+        # every other BASELINE config, the expanded-head cache of the reference's engine, head_dim 64
+        legs = {}
+        for name in ("cfg1", "cfg2x", "cfg2xs", "cfg2d64", "cfg4d", "cfg5"):
+            if name != args.workload:
+                legs[name] = decode_leg(name, hbm_budget_gb=args.hbm_budget_gb if name == "cfg5" else None,
+                                        cpu=(name == "cfg1" and not args.no_cpu_baseline))
+        result["workloads"] = legs
+        result["cfg4_mixed_step"] = cfg4_mixed_step()
+        result["prefill_sized"] = append_gather_rates()
+        result["chunked_prefill"] = prefill_rate()
+        result["chunked_prefill_expanded_heads"] = prefill_rate(name="cfg3x")
+        result["chunked_prefill_head_dim_64"] = prefill_rate(name="cfg3d64")
+        result["chunked_prefill_fp32"] = prefill_rate(name="cfg3f32")
+        result["chunked_prefill_one_sequence"] = prefill_rate(name="cfg3one")
+        result["decode_small_batch"] = small_batch_decode()
     print(json.dumps(result))
     return 0
 
