@@ -4,12 +4,18 @@
 // PagedKVCache.assign_prefill_no_paging (:364-393): a pure byte copy of each
 // (token, head) row to pool[h, page_table[batch_idx, pos / P] * P + pos % P, :].
 //
-// HBM-bound.  A row is D * elem bytes (256 B at D = 128 bf16); it is moved as
-// 16-byte vectors, one vector of K and one of V per lane, four such pairs in
-// flight per lane.  Lanes run fastest over the bytes of a row, then over tokens
-// of one head, so a wavefront writes consecutive slots of a page as one
-// contiguous run and reads whole 256-byte rows of the source.  The slot is
-// computed in the kernel from the page table, there is no separate slot-mapping pass.
+// HBM-bound.  A row is D * elem bytes (256 B at D = 128 bf16); it is moved as 16-byte
+// vectors (8/4/2-byte ones when alignment asks for it), ONE vector of K and one of V per lane.
+// The lanes of a launch run over the source in its memory order: for the [T, H, D] rows the
+// model produces (reference model.py:116-119) over (token, head, chunk), so that consecutive
+// lanes read consecutive bytes and each row is written as one 256-byte piece of its page.
+// Measured at 32768 tokens x 16 heads (537 MB moved; a plain copy of that size takes 90 us):
+// 98-102 us whatever the buffers' placement in memory.  More vectors per lane are slower (2: 104 us,
+// 4: 107 us, 8: 117 us); a grid of (row tiles, heads) with lanes over the tokens of one head, which
+// reads 256-byte pieces 4 KiB apart, takes 93 us or 115 us depending on where the allocator
+// placed the buffers (the same process sees both), and dealing those workgroups so that the heads
+// of a row tile run back to back on one XCD gives 98-103 us.
+// The slot is computed in the kernel from the page table, there is no separate slot-mapping pass.
 // Loads and stores are non-temporal: the rows are touched once and should not displace
 // cache lines other kernels reuse.
 #include "fp_common.h"
@@ -44,63 +50,73 @@ struct AppendArgs {
 };
 
 constexpr int kThreads = 256;
-constexpr int kItems = 4;  // (K, V) vector pairs per lane
 
-template <typename Vec>
-__global__ __launch_bounds__(kThreads) void kv_append_kernel(const AppendArgs a) {
-  const int h = blockIdx.y;
-  const int64_t items = static_cast<int64_t>(a.n_tok) * a.chunks;
-  const int64_t base = static_cast<int64_t>(blockIdx.x) * (kThreads * kItems) + threadIdx.x;
-
-  Vec kreg[kItems], vreg[kItems];
-  int64_t dst[kItems];
-
-#pragma unroll
-  for (int j = 0; j < kItems; ++j) {
-    const int64_t i = base + static_cast<int64_t>(j) * kThreads;
-    dst[j] = -1;
-    if (i >= items) continue;
-    const int tok = static_cast<int>(i / a.chunks);
-    const int c = static_cast<int>(i - static_cast<int64_t>(tok) * a.chunks);
-    int t = tok, s = 0;
-    if (a.S != 1) {
-      t = tok / a.S;
-      s = tok - t * a.S;
-    }
-    const int64_t ko = t * a.ks_t + h * a.ks_h + s * a.ks_s + static_cast<int64_t>(c) * sizeof(Vec);
-    const int64_t vo = t * a.vs_t + h * a.vs_h + s * a.vs_s + static_cast<int64_t>(c) * sizeof(Vec);
-    kreg[j] = __builtin_nontemporal_load(reinterpret_cast<const Vec*>(a.k + ko));
-    vreg[j] = __builtin_nontemporal_load(reinterpret_cast<const Vec*>(a.v + vo));
-
-    const int64_t b = a.batch_idx[t];
-    const int64_t pos = fp::load_index(a.input_pos, tok, a.pos_i64);
-    if (b < 0 || b >= a.max_batch || pos < 0) continue;
-    int64_t blk;
-    int off;
-    a.pd.split(pos, blk, off);
-    if (blk >= a.n_pages) continue;
-    int64_t page = a.page_table[b * a.pt_row_stride + blk];
-    if (a.clamp_negative && page < 0) page = 0;
-    int64_t slot = page * a.pd.page_size + off;
-    if (slot < 0) slot += a.n_slots;  // negative index counts from the end of the slot axis
-    if (slot < 0 || slot >= a.n_slots) continue;
-    dst[j] = (static_cast<int64_t>(h) * a.n_slots + slot) * a.row_bytes + static_cast<int64_t>(c) * sizeof(Vec);
+// One 16-byte vector of K and one of V per lane.  kTokenMajor: lanes run over (token, head, chunk), the
+// order of a [T, H, D] source, so a load instruction reads consecutive source bytes and every row leaves
+// as one 256-byte piece; otherwise grid.y = head and lanes run over (token, chunk), the order of a
+// [H, T, D] source, where source and destination are both contiguous per head.  Idx = uint32_t whenever
+// the item count allows (one division per lane instead of a 64-bit one).
+template <typename Vec, bool kTokenMajor, typename Idx>
+__global__ __launch_bounds__(kThreads) void kv_append_kernel(const AppendArgs a, int H) {
+  const Idx per_tok = kTokenMajor ? static_cast<Idx>(H) * a.chunks : static_cast<Idx>(a.chunks);
+  const Idx items = static_cast<Idx>(a.n_tok) * per_tok;
+  const Idx i = static_cast<Idx>(blockIdx.x) * kThreads + threadIdx.x;
+  if (i >= items) return;
+  const int tok = static_cast<int>(i / per_tok);
+  int c = static_cast<int>(i - static_cast<Idx>(tok) * per_tok);
+  int h = blockIdx.y;
+  if (kTokenMajor) {
+    h = c / a.chunks;
+    c -= h * a.chunks;
   }
-
-#pragma unroll
-  for (int j = 0; j < kItems; ++j) {
-    if (dst[j] < 0) continue;
-    __builtin_nontemporal_store(kreg[j], reinterpret_cast<Vec*>(a.pool_k + dst[j]));
-    __builtin_nontemporal_store(vreg[j], reinterpret_cast<Vec*>(a.pool_v + dst[j]));
+  int t = tok, s = 0;
+  if (a.S != 1) {
+    t = tok / a.S;
+    s = tok - t * a.S;
   }
+  const int64_t ko = t * a.ks_t + h * a.ks_h + s * a.ks_s + static_cast<int64_t>(c) * sizeof(Vec);
+  const int64_t vo = t * a.vs_t + h * a.vs_h + s * a.vs_s + static_cast<int64_t>(c) * sizeof(Vec);
+  const Vec kreg = __builtin_nontemporal_load(reinterpret_cast<const Vec*>(a.k + ko));
+  const Vec vreg = __builtin_nontemporal_load(reinterpret_cast<const Vec*>(a.v + vo));
+
+  const int64_t b = a.batch_idx[t];
+  const int64_t pos = fp::load_index(a.input_pos, tok, a.pos_i64);
+  if (b < 0 || b >= a.max_batch || pos < 0) return;
+  int64_t blk;
+  int off;
+  a.pd.split(pos, blk, off);
+  if (blk >= a.n_pages) return;
+  int64_t page = a.page_table[b * a.pt_row_stride + blk];
+  if (a.clamp_negative && page < 0) page = 0;
+  int64_t slot = page * a.pd.page_size + off;
+  if (slot < 0) slot += a.n_slots;  // negative index counts from the end of the slot axis
+  if (slot < 0 || slot >= a.n_slots) return;
+  const int64_t dst = (static_cast<int64_t>(h) * a.n_slots + slot) * a.row_bytes + static_cast<int64_t>(c) * sizeof(Vec);
+  __builtin_nontemporal_store(kreg, reinterpret_cast<Vec*>(a.pool_k + dst));
+  __builtin_nontemporal_store(vreg, reinterpret_cast<Vec*>(a.pool_v + dst));
 }
 
 template <typename Vec>
-void launch(const AppendArgs& a, int H, hipStream_t stream) {
-  const int64_t items = static_cast<int64_t>(a.n_tok) * a.chunks;
-  const int64_t per_block = kThreads * kItems;
-  dim3 grid(static_cast<unsigned>((items + per_block - 1) / per_block), static_cast<unsigned>(H));
-  hipLaunchKernelGGL(kv_append_kernel<Vec>, grid, dim3(kThreads), 0, stream, a);
+int launch(const AppendArgs& a, int H, hipStream_t stream) {
+  // the source's memory order decides which index runs fastest across the lanes
+  const bool token_major = a.ks_h <= a.ks_t && a.vs_h <= a.vs_t;
+  const int64_t per_grid_row = static_cast<int64_t>(a.n_tok) * a.chunks * (token_major ? H : 1);
+  const int64_t blocks = (per_grid_row + kThreads - 1) / kThreads;
+  if (blocks > INT32_MAX) return fp::fail(FP_ERR_UNSUPPORTED, "fp_kv_append: more than 2^31-1 workgroups");
+  const bool narrow = per_grid_row + kThreads < (1ll << 32);
+  dim3 grid(static_cast<unsigned>(blocks), token_major ? 1u : static_cast<unsigned>(H));
+  if (token_major) {
+    if (narrow)
+      hipLaunchKernelGGL((kv_append_kernel<Vec, true, uint32_t>), grid, dim3(kThreads), 0, stream, a, H);
+    else
+      hipLaunchKernelGGL((kv_append_kernel<Vec, true, int64_t>), grid, dim3(kThreads), 0, stream, a, H);
+  } else {
+    if (narrow)
+      hipLaunchKernelGGL((kv_append_kernel<Vec, false, uint32_t>), grid, dim3(kThreads), 0, stream, a, H);
+    else
+      hipLaunchKernelGGL((kv_append_kernel<Vec, false, int64_t>), grid, dim3(kThreads), 0, stream, a, H);
+  }
+  return FP_OK;
 }
 
 }  // namespace
@@ -148,11 +164,13 @@ extern "C" int fp_kv_append(void* pool_k, void* pool_v, const void* k, const voi
   a.chunks = a.row_bytes / vec;
 
   hipStream_t st = static_cast<hipStream_t>(stream);
+  int rc;
   switch (vec) {
-    case 16: launch<v4u>(a, H, st); break;
-    case 8: launch<v2u>(a, H, st); break;
-    case 4: launch<uint32_t>(a, H, st); break;
-    default: launch<uint16_t>(a, H, st); break;
+    case 16: rc = launch<v4u>(a, H, st); break;
+    case 8: rc = launch<v2u>(a, H, st); break;
+    case 4: rc = launch<uint32_t>(a, H, st); break;
+    default: rc = launch<uint16_t>(a, H, st); break;
   }
+  if (rc != FP_OK) return rc;
   return fp::check_launch("fp_kv_append");
 }

@@ -37,54 +37,46 @@ struct GatherArgs {
 };
 
 constexpr int kThreads = 256;
-constexpr int kItems = 4;
-
+// One 16-byte vector per lane: more vectors per lane measured slower (32768 tokens x 16 heads,
+// 268 MB moved: 46 us with one, 47 with two, 49 with four).
 template <typename Vec>
 __global__ __launch_bounds__(kThreads) void kv_gather_kernel(const GatherArgs a) {
   const int h = blockIdx.y;
   const int b = blockIdx.z;
   const int64_t items = static_cast<int64_t>(a.max_len) * a.chunks;
-  const int64_t base = static_cast<int64_t>(blockIdx.x) * (kThreads * kItems) + threadIdx.x;
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (i >= items) return;
 
   int64_t len = fp::load_index(a.seq_lens, b, a.len_i64);
   const int64_t row = a.batch_idx[b];
   if (row < 0 || row >= a.max_batch) len = 0;
   if (len > a.max_len) len = a.max_len;
 
-  Vec reg[kItems];
-  int64_t dst[kItems];
-#pragma unroll
-  for (int j = 0; j < kItems; ++j) {
-    const int64_t i = base + static_cast<int64_t>(j) * kThreads;
-    dst[j] = -1;
-    reg[j] = Vec(0);
-    if (i >= items) continue;
-    const int t = static_cast<int>(i / a.chunks);
-    const int c = static_cast<int>(i - static_cast<int64_t>(t) * a.chunks);
-    dst[j] = b * a.os_b + h * a.os_h + t * a.os_t + static_cast<int64_t>(c) * sizeof(Vec);
-    if (t >= len) continue;
+  const int t = i < (1ll << 32) ? static_cast<int>(static_cast<uint32_t>(i) / static_cast<uint32_t>(a.chunks))
+                                : static_cast<int>(i / a.chunks);
+  const int c = static_cast<int>(i - static_cast<int64_t>(t) * a.chunks);
+  const int64_t dst = b * a.os_b + h * a.os_h + t * a.os_t + static_cast<int64_t>(c) * sizeof(Vec);
+  Vec reg = Vec(0);
+  if (t < len) {
     int64_t blk;
     int off;
     a.pd.split(t, blk, off);
-    if (blk >= a.n_pages) continue;
-    const int64_t page = a.page_table[row * a.pt_row_stride + blk];
-    const int64_t slot = page * a.pd.page_size + off;
-    if (slot < 0 || slot >= a.n_slots) continue;
-    const int64_t src = (static_cast<int64_t>(h) * a.n_slots + slot) * a.row_bytes + static_cast<int64_t>(c) * sizeof(Vec);
-    reg[j] = __builtin_nontemporal_load(reinterpret_cast<const Vec*>(a.pool + src));
+    if (blk < a.n_pages) {
+      const int64_t page = a.page_table[row * a.pt_row_stride + blk];
+      const int64_t slot = page * a.pd.page_size + off;
+      if (slot >= 0 && slot < a.n_slots) {
+        const int64_t src = (static_cast<int64_t>(h) * a.n_slots + slot) * a.row_bytes + static_cast<int64_t>(c) * sizeof(Vec);
+        reg = __builtin_nontemporal_load(reinterpret_cast<const Vec*>(a.pool + src));
+      }
+    }
   }
-#pragma unroll
-  for (int j = 0; j < kItems; ++j) {
-    if (dst[j] < 0) continue;
-    __builtin_nontemporal_store(reg[j], reinterpret_cast<Vec*>(a.out + dst[j]));
-  }
+  __builtin_nontemporal_store(reg, reinterpret_cast<Vec*>(a.out + dst));
 }
 
 template <typename Vec>
 void launch_gather(const GatherArgs& a, int B, int H, hipStream_t stream) {
   const int64_t items = static_cast<int64_t>(a.max_len) * a.chunks;
-  const int64_t per_block = kThreads * kItems;
-  dim3 grid(static_cast<unsigned>((items + per_block - 1) / per_block), static_cast<unsigned>(H),
+  dim3 grid(static_cast<unsigned>((items + kThreads - 1) / kThreads), static_cast<unsigned>(H),
             static_cast<unsigned>(B));
   hipLaunchKernelGGL(kv_gather_kernel<Vec>, grid, dim3(kThreads), 0, stream, a);
 }
