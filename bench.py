@@ -533,6 +533,11 @@ def append_gather_rates(steps: int = 20, T: int = 32768, H: int = 16, D: int = 1
     bytes_r = (T * (H + 2 * Hkv) * D * e + T * (D // 4) * 8 + T * H * (D // 4) * 8
                + T * H * D * e + 2 * T * H * D * e + 16 * T)
     return {"tokens": T, "heads": H, "head_dim": D,
+            "algorithmic_bytes": {"kv_append": bytes_a, "kv_gather": bytes_g, "qkv_norm_rope_append": bytes_r},
+            # HBM bytes per launch from the rocprofv3 FETCH_SIZE / WRITE_SIZE summaries under profiles/
+            "traffic": {"kv_append": profiled_traffic("kv_append", f"{T}x{H}"),
+                        "kv_gather": profiled_traffic("kv_gather", f"{T}x{H}"),
+                        "qkv_norm_rope_append": profiled_traffic("qkv_rope_append", f"{T}x{H}")},
             "qkv_norm_rope_append_ms": ms_r, "qkv_norm_rope_append_gbps": bytes_r / (ms_r * 1e-3) / 1e9,
             "qkv_norm_rope_append_frac_of_peak": bytes_r / (ms_r * 1e-3) / 1e9 / HBM_PEAK_GBPS,
             "kv_append_ms": ms_a, "kv_append_gbps": bytes_a / (ms_a * 1e-3) / 1e9,
