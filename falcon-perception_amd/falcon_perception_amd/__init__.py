@@ -13,7 +13,7 @@ from .paged_attention import PagedKVCache  # noqa: F401
 __all__ = ["KVCacheBase", "PagedKVCache", "attention", "kv_cache", "ops", "paged_attention", "install"]
 
 
-def install() -> None:
+def install(kv_rep: int = 1) -> None:
     """Serve the reference's module names from this package.
 
     After `install()`, `import falcon_perception.paged_attention`,
@@ -21,9 +21,19 @@ def install() -> None:
     modules here, so the reference's `model.py`, `paged_inference.py` and
     `paged_ocr_inference.py` bind these implementations at import time without
     any change to their source.  Call it before importing those modules.
+
+    `kv_rep` = n_heads // n_kv_heads of the model to be served (2 for every variant of the
+    reference, `falcon_perception/__init__.py:36-40`) tells every cache created afterwards that
+    the V heads it is given are that many identical copies per kv head, which is what the
+    reference's `repeat_kv` hands to `insert_kv` (`model.py:112-116`): decode then reads V once
+    per group.  The engine builds its cache with `n_heads` heads (`paged_inference.py:321-330`)
+    and never says so itself; left at 1, every cached head is read in full.
     """
     import sys
 
+    if kv_rep < 1:
+        raise ValueError("kv_rep must be at least 1")
+    PagedKVCache.default_kv_rep = int(kv_rep)
     sys.modules["falcon_perception.kv_cache"] = kv_cache
     sys.modules["falcon_perception.paged_attention"] = paged_attention
     sys.modules["falcon_perception.attention"] = attention

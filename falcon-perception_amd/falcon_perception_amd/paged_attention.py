@@ -52,6 +52,8 @@ class PagedKVCache(KVCacheBase):
     table (`get_mask_mod`, the element mask of the reference's flex kernels) is then unavailable.
     """
 
+    default_kv_rep = 1  # kv_rep of caches created from now on, see `falcon_perception_amd.install`
+
     def __init__(self, n_pages: int, page_size: int, max_batch_size: int, n_heads: int, head_dim: int,
                  num_layers: int, dtype: torch.dtype, device: str | torch.device = "cuda",
                  max_blocks_per_seq: int | None = None):
@@ -78,8 +80,10 @@ class PagedKVCache(KVCacheBase):
         self.kv_cache = torch.zeros(self.kv_shape, dtype=dtype, device=device)
 
         # 1, or n_heads // n_kv_heads when the cached V heads are plain copies inside a group (the model's
-        # repeat_kv, model.py:112-113): the decode kernel then reads V once per group.  Off unless set.
-        self.kv_rep = 1
+        # repeat_kv, model.py:112-113): the decode kernel then reads V once per group.  Taken from the class
+        # default (`falcon_perception_amd.install(kv_rep=...)` sets it for an engine that is not edited) when
+        # it divides this cache's head count.
+        self.kv_rep = self.default_kv_rep if n_heads % self.default_kv_rep == 0 else 1
 
         # what the attention callables need from the step in flight
         self.last_decode_step: StepMeta | None = None
@@ -162,6 +166,17 @@ class PagedKVCache(KVCacheBase):
         else:
             self.last_prefill_step = StepMeta(layer_id, input_pos, batch_idx)
         return q, self.kv_cache[layer_id, 0], self.kv_cache[layer_id, 1]
+
+    def v_copies_are_identical(self, layer_id: int = 0) -> bool:
+        """Whether the V plane of a layer really holds `kv_rep` identical heads per group (bit for bit, over
+        the whole pool): the condition under which decoding with `kv_rep` > 1 equals the plain read.  A check
+        for bring-up; it reads the plane and waits for the result."""
+        if self.kv_rep == 1:
+            return True
+        v = self.kv_cache[layer_id, 1, 0]
+        groups = v.view(v.shape[0] // self.kv_rep, self.kv_rep, *v.shape[1:])
+        bits = groups.view(torch.int16 if v.element_size() == 2 else torch.int32)
+        return bool((bits == bits[:, :1]).all())
 
     # --------------------------------------------------------------- allocator
     @property

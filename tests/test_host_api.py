@@ -260,3 +260,22 @@ def test_prefill_row_limit_survives_inference_mode():
         pos.add_(100)  # the engine's next step may reuse the buffer
         assert m.row_limit(pos, 0).tolist() == [111, 115, 115, 115, 115, 116]
         assert m.row_limit(torch.arange(6)[None], 1).tolist() == [1, 5, 5, 5, 5, 6]
+
+
+def test_install_serves_the_reference_module_names_and_sets_kv_rep(monkeypatch):
+    monkeypatch.setattr(PagedKVCache, "default_kv_rep", 1)
+    for name in ("falcon_perception.kv_cache", "falcon_perception.paged_attention", "falcon_perception.attention"):
+        monkeypatch.delitem(sys.modules, name, raising=False)
+    fpa.install(kv_rep=2)
+    import importlib
+
+    assert importlib.import_module("falcon_perception.paged_attention").PagedKVCache is PagedKVCache
+    assert importlib.import_module("falcon_perception.attention").compiled_flex_attn_decode is A.compiled_flex_attn_decode
+    # what the engine builds (paged_inference.py:321-330): n_heads cached heads; the cache now knows the V copies
+    c = PagedKVCache(8, 4, 4, 16, 8, 1, torch.float32, device="cpu")
+    assert c.kv_rep == 2 and c.v_copies_are_identical()
+    c.kv_cache[0, 1, 0, 1, 5] = 1.0  # head 1 no longer equals head 0
+    assert not c.v_copies_are_identical()
+    assert PagedKVCache(8, 4, 4, 3, 8, 1, torch.float32, device="cpu").kv_rep == 1  # 3 heads: no groups of 2
+    with pytest.raises(ValueError):
+        fpa.install(kv_rep=0)
