@@ -119,3 +119,35 @@ def test_shared_v_and_sink_gate_through_the_even_cut():
     gate = 1.0 / (1.0 + np.exp(f64(sinks)[None, :, None] - f64(lse)))
     np.testing.assert_allclose(f64(gated), f64(out) * gate[..., None], atol=atol, rtol=rtol)
     assert not f64(out)[0].any() and np.isneginf(f64(lse)[0]).all()  # the sequence without keys
+
+
+def test_a_cache_that_knows_its_v_copies_decodes_through_the_reference_call():
+    """`install(kv_rep=2)` gives every new cache kv_rep = 2; the unchanged call sequence of the reference
+    (insert_kv with expanded K/V, compiled_flex_attn_decode on the returned pool views) then reads V once per
+    group and returns what the plain read returns."""
+    from torch.nn.attention.flex_attention import AuxRequest
+
+    from falcon_perception_amd import attention as A
+
+    dtype, P, rep = torch.bfloat16, 32, 2
+    lens = [5, 64, 300, 31]
+    st, Hq = expanded_state(57, rep, dtype, P, lens)
+    cache = st.cache
+    B = len(lens)
+    bidx = torch.tensor(st.slots, dtype=torch.int64, device=DEV)
+    pos = torch.tensor(lens, dtype=torch.int32, device=DEV)
+    k = randn(st.gen, (B, Hq, 1, 128), dtype).to(DEV)
+    v = randn(st.gen, (B, Hq // rep, 1, 128), dtype).repeat_interleave(rep, dim=1).to(DEV)
+    q = randn(st.gen, (B, Hq, 1, 128), dtype).to(DEV)
+    logical = cache.create_causal_blockmask(B=B, L=512)
+    mask = cache.convert_logical_block_mask(logical, bidx)  # the kernel takes positions from the step, not the mask
+    results = {}
+    for r in (1, rep):
+        cache.kv_rep = r
+        K, V = cache.insert_kv(0, k, v, input_pos=pos.view(B, 1), batch_idx=bidx)
+        out, aux = A.compiled_flex_attn_decode(q, K, V, block_mask=mask, return_aux=AuxRequest(lse=True))
+        results[r] = (out.clone(), aux.lse.clone())
+    assert cache.v_copies_are_identical()
+    assert torch.equal(results[1][0], results[rep][0]) and torch.equal(results[1][1], results[rep][1])
+    eo, el = O.decode_attention(f64(q), f64(K[0]), f64(V[0]), st.mirror.page_table, st.slots, np.array(lens), P)
+    np.testing.assert_allclose(f64(results[rep][0]), eo, atol=2e-2, rtol=1e-2)
