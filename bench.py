@@ -55,16 +55,21 @@ DTYPES = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
 def profiled_traffic(kernel: str, workload: str) -> float | None:
     """HBM bytes per launch of `kernel` at `workload` as a rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE pair
     measured them (each scaled by the same counter on a plain copy of known size): the line
-    `traffic_bytes_per_launch = N` of profiles/<kernel>_<workload>_hbm_traffic.md, None when no such
+    `traffic_bytes_per_launch = N` of profiles/<kernel>_<workload>_hbm_traffic.md, or the line
+    `traffic_bytes_per_launch[<workload>] = N` of profiles/<kernel>_hbm_traffic.md; None when no such
     summary has been recorded."""
     import re
 
-    path = os.path.join(ROOT, "profiles", f"{kernel}_{workload}_hbm_traffic.md")
-    try:
-        m = re.search(r"traffic_bytes_per_launch\s*=\s*([0-9.eE+]+)", open(path).read())
-    except OSError:
-        return None
-    return float(m.group(1)) if m else None
+    for name, pattern in ((f"{kernel}_{workload}_hbm_traffic.md", r"traffic_bytes_per_launch\s*=\s*([0-9.eE+]+)"),
+                          (f"{kernel}_hbm_traffic.md",
+                           r"traffic_bytes_per_launch\[" + re.escape(workload) + r"\]\s*=\s*([0-9.eE+]+)")):
+        try:
+            m = re.search(pattern, open(os.path.join(ROOT, "profiles", name)).read())
+        except OSError:
+            continue
+        if m:
+            return float(m.group(1))
+    return None
 
 
 @dataclass
@@ -360,9 +365,11 @@ def warm_clocks(fn, seconds: float = 0.2) -> None:
         torch.cuda.synchronize()
 
 
-def event_ms(fn, steps: int) -> float:
-    """Device ms per call of `fn`: HIP events on the stream the kernels run on around every call, median of
-    at least 20 calls."""
+def event_ms(fn, steps: int, batch: int = 1) -> float:
+    """Device ms per call of `fn`: HIP events on the stream the kernels run on, median of at least 20
+    samples.  A sample brackets `batch` back-to-back calls (result divided by `batch`): around a single
+    launch the two event markers themselves add 1.5-4 us to what the kernel trace of rocprofv3 reports for
+    the kernel, around ten launches a tenth of that."""
     warm_clocks(fn)
     n = max(steps, 20)
     stream = torch.cuda.current_stream()
@@ -370,10 +377,11 @@ def event_ms(fn, steps: int) -> float:
     ends = [torch.cuda.Event(enable_timing=True) for _ in range(n)]
     for i in range(n):
         starts[i].record(stream)
-        fn()
+        for _ in range(batch):
+            fn()
         ends[i].record(stream)
     torch.cuda.synchronize()
-    return statistics.median(s.elapsed_time(e) for s, e in zip(starts, ends))
+    return statistics.median(s.elapsed_time(e) for s, e in zip(starts, ends)) / batch
 
 
 def graph_ms(fn, steps: int) -> float:
@@ -606,7 +614,7 @@ def decode_leg(name: str, steps: int = 20, hbm_budget_gb: float | None = None, c
     case = make_decode_case(name, hbm_budget_gb=hbm_budget_gb)
     c = case.cfg
     ms_step = time_steps(case.run_fused, steps, 5, samples=11)
-    ms_partial = event_ms(lambda: case.attend("partial"), steps)
+    ms_partial = event_ms(lambda: case.attend("partial"), steps, batch=10)
     alg_decode, alg_append = case.bytes_decode(), case.bytes_append()
     gbps = (alg_decode + alg_append) / (ms_step * 1e-3) / 1e9
     kernel_gbps = alg_decode / (ms_partial * 1e-3) / 1e9
@@ -831,7 +839,7 @@ def main() -> int:
     ms_gated = time_steps(case.run_fused_gated, args.steps, args.warmup, samples=5)
     ms_graph = graph_ms(case.run_fused, args.steps)
     ms_decode = event_ms(case.attend, args.steps)
-    ms_partial = event_ms(lambda: case.attend("partial"), args.steps)  # the dominant kernel alone
+    ms_partial = event_ms(lambda: case.attend("partial"), args.steps, batch=10)  # the dominant kernel alone
     ms_merge = event_ms(lambda: case.attend("merge"), args.steps)
     ms_append = event_ms(case.append, args.steps)
     case.attend()
