@@ -471,8 +471,8 @@ def append_gather_rates(steps: int = 20, T: int = 32768, H: int = 16, D: int = 1
     for _ in range(3):
         do_append()
         do_gather()
-    ms_a = event_ms(do_append, steps)
-    ms_g = event_ms(do_gather, steps)
+    ms_a = event_ms(do_append, steps, batch=5)
+    ms_g = event_ms(do_gather, steps, batch=5)
     e = 2
     bytes_a = 2 * T * (2 * H * D * e) + 8 * T
     bytes_g = 2 * T * (H * D * e)
@@ -514,8 +514,8 @@ def append_gather_rates(steps: int = 20, T: int = 32768, H: int = 16, D: int = 1
 
     for _ in range(len(rings)):
         do_append_cold()
-    ms_cold = event_ms(do_append_cold, 3 * len(rings))
-    ms_g_cold = event_ms(do_gather_cold, 3 * len(rings))
+    ms_cold = event_ms(do_append_cold, 20, batch=len(rings))
+    ms_g_cold = event_ms(do_gather_cold, 20, batch=len(rings))
     del rings
 
     # QK norm + rotary embedding + insert in one launch (reference model.py:110-119 + the append):
@@ -536,7 +536,7 @@ def append_gather_rates(steps: int = 20, T: int = 32768, H: int = 16, D: int = 1
 
     for _ in range(3):
         do_rope()
-    ms_r = event_ms(do_rope, steps)
+    ms_r = event_ms(do_rope, steps, batch=5)
     # read q, k, v rows and both angle tables once, write q and the expanded K and V rows, token indices
     bytes_r = (T * (H + 2 * Hkv) * D * e + T * (D // 4) * 8 + T * H * (D // 4) * 8
                + T * H * D * e + 2 * T * H * D * e + 16 * T)
@@ -565,7 +565,7 @@ def prefill_rate(steps: int = 10, name: str = "cfg3") -> dict:
     case.append()
     for _ in range(3):
         case.attend()
-    ms = event_ms(case.attend, steps)
+    ms = event_ms(case.attend, steps, batch=4)
     ms_a = event_ms(case.append, steps)
     tf = case.flops() / (ms * 1e-3) / 1e12
     what = {"cfg3": "cfg3: 8 sequences, paged prefix U[256,4096], 512-token chunk each, 16 q / 8 kv heads, D 128",

@@ -16,11 +16,10 @@
 // HBM / launch bound.  A group of D * elem / 16 lanes holds a row in one 16-byte vector per lane.  For the
 // model's shapes (Hq / Hkv in {1, 2, 4, 8}, head_dim 64 or 128) a group owns one (token, kv head): the query
 // rows of the kv head, its K row and its V row, so that the per-head angles are fetched once for the query
-// row and the K replica that share them (32768 tokens, 16 q / 8 kv heads: 129 us against 154 us row by
-// row, where the angle table was fetched twice).  Other shapes go row by row: one group per source row
-// (token, head).  Either way groups run token-fastest inside a head so that a wavefront stores consecutive
-// pool slots; a K row is normalised once and rotated once per replica (the 2D angles differ per head), a V
-// row is stored n_rep times.
+// row and the K replica that share them (32768 tokens, 16 q / 8 kv heads: 134 us against 154 us row by
+// row, where the angle table was fetched twice); the groups run over the source in its memory order.  Other
+// shapes go row by row: one group per source row (token, head), token-fastest inside a head.  A K row is
+// normalised once and rotated once per replica (the 2D angles differ per head), a V row is stored n_rep times.
 #include "fp_common.h"
 
 #include <hip/hip_bf16.h>
@@ -52,6 +51,7 @@ struct RopeArgs {
   int64_t n_slots;
   float eps;
   int clamp_negative;
+  int order;  // groups of the (token, kv head) kernel: 1 = kv heads of a token fastest, 0 = tokens of a kv head fastest
 };
 
 struct F32 {
@@ -213,7 +213,10 @@ __global__ __launch_bounds__(kThreads) void qkv_rope_append_kernel(const RopeArg
 // its K row and its V row.  With per-head 2D angles, the K replica of head h and the query row of head h
 // rotate by the same angles, so a group fetches every angle row ONCE (the row-per-group kernel above reads
 // the [T, Hq, D/4] table twice, 134 MB of 814 MB at 32768 tokens x 16 heads, because query rows and K rows
-// of a head are handled by workgroups far apart in time).  Groups run token-fastest inside a kv head.
+// of a head are handled by workgroups far apart in time).  Groups run over the source in its memory order
+// (a.order): for the projection output [T, heads, D] the kv heads of a token run fastest, so a workgroup reads
+// whole 8 KiB token rows.  Tokens fastest inside a kv head measured 129 us or 141 us at 32768 tokens depending
+// on where the allocator had placed the buffers, kv heads fastest 134 us either way.
 template <typename E, int TPR, int NQ>
 __global__ __launch_bounds__(kThreads) void qkv_rope_group_kernel(const RopeArgs a) {
   constexpr int EPV = E::kEpv;
@@ -222,9 +225,9 @@ __global__ __launch_bounds__(kThreads) void qkv_rope_group_kernel(const RopeArgs
   constexpr int kRows = kThreads / TPR;
   const int sub = threadIdx.x % TPR;  // this lane's 16-byte vector inside a row
   const int64_t uid = static_cast<int64_t>(blockIdx.x) * kRows + threadIdx.x / TPR;
-  const int g = static_cast<int>(uid / a.T);  // kv head
-  const int t = static_cast<int>(uid - static_cast<int64_t>(g) * a.T);
-  const bool live = g < a.Hkv;  // lanes of one group agree; dead groups still take part in the shuffles
+  const int g = a.order ? static_cast<int>(uid % a.Hkv) : static_cast<int>(uid / a.T);  // kv head
+  const int t = a.order ? static_cast<int>(uid / a.Hkv) : static_cast<int>(uid - static_cast<int64_t>(g) * a.T);
+  const bool live = a.order ? t < a.T : g < a.Hkv;  // lanes of one group agree; dead groups still take part in the shuffles
 
   // every load of the group is requested before the first use
   v4u rq[NQ];
@@ -423,7 +426,10 @@ extern "C" int fp_qkv_norm_rope_append(const void* xq, const void* xk, const voi
              freqs_cis, freqs_cis_2d, static_cast<char*>(q_out), qo_stride_t * eb, qo_stride_h * eb,
              static_cast<char*>(pool_k), static_cast<char*>(pool_v), page_table, pt_row_stride, batch_idx, input_pos,
              pos_index_type == FP_INDEX_I64, T, Hq, Hkv, H_pool / Hkv, fp::PageDiv(page_size), n_pages, max_batch,
-             n_slots, eps, clamp_negative};
+             n_slots, eps, clamp_negative,
+             // the groups run over the source in its memory order: the kv heads of a token next to each other for the
+             // [T, heads, D] projection output
+             (q_stride_h <= q_stride_t && k_stride_h <= k_stride_t && v_stride_h <= v_stride_t) ? 1 : 0};
   hipStream_t st = static_cast<hipStream_t>(stream);
   int rc;
   if (dtype == FP_DTYPE_F32) rc = launch<F32>(a, D, st);
