@@ -279,3 +279,21 @@ def test_install_serves_the_reference_module_names_and_sets_kv_rep(monkeypatch):
     assert PagedKVCache(8, 4, 4, 3, 8, 1, torch.float32, device="cpu").kv_rep == 1  # 3 heads: no groups of 2
     with pytest.raises(ValueError):
         fpa.install(kv_rep=0)
+
+
+def test_bench_reads_traffic_from_the_profiles_and_refuses_several_gpus():
+    import subprocess
+
+    import bench
+
+    # the decode workloads share one summary (a line per workload), the other kernels have a file each
+    for wl in ("cfg1", "cfg2", "cfg2x", "cfg2xs", "cfg2d64", "cfg4d", "cfg5"):
+        t = bench.profiled_traffic("paged_decode", wl)
+        assert t is not None and t > 1e6, wl
+    for kernel in ("kv_append", "kv_gather", "qkv_rope_append"):
+        assert bench.profiled_traffic(kernel, "32768x16") > 2.6e8
+    assert bench.profiled_traffic("paged_decode", "no_such_workload") is None
+    # traffic must not fall below the algorithmic bytes it is compared with (cfg2: 666.07 MB)
+    assert 666.0e6 < bench.profiled_traffic("paged_decode", "cfg2") < 1.05 * 666.1e6
+    res = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert res.returncode == 2 and "ONE GPU" in res.stderr and not res.stdout.strip()
