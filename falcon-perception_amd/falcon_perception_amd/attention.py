@@ -241,8 +241,11 @@ def compiled_flex_attn_decode(q: Tensor, k: Tensor, v: Tensor, score_mod=None, b
     kv_rep = getattr(cache, "kv_rep", 1)
     wg_heads = k.shape[1] // kv_rep  # workgroups per sequence and split
     workspace, split_tokens = cache.decode_launch(q.shape[0], q.shape[1], q.shape[3], block_mask.max_context, wg_heads)
+    # the pool views insert_kv returned, as planes [H, N, D]: the cache keeps both forms of every layer
+    pools = cache._pools[step.layer_id]
+    pool_k, pool_v = cache._planes[step.layer_id] if (k is pools[0] and v is pools[1]) else (k[0], v[0])
     out, lse = ops.paged_decode(
-        q, k[0], v[0], cache.page_table, block_mask.batch_idx, step.input_pos,
+        q, pool_k, pool_v, cache.page_table, block_mask.batch_idx, step.input_pos,
         cache.page_size, block_mask.max_context, scale=scale,
         workspace=workspace, split_tokens=split_tokens, sinks=sinks, kv_rep=kv_rep,
     )
@@ -272,8 +275,7 @@ def compiled_flex_attn_prefill(q: Tensor, k: Tensor, v: Tensor, score_mod=None, 
     step = cache.last_prefill_step
     if step is None:
         raise RuntimeError("paged prefill attention called before PagedKVCache.insert_kv for this step")
-    pool_k = cache.kv_cache[step.layer_id, 0, 0]
-    pool_v = cache.kv_cache[step.layer_id, 1, 0]
+    pool_k, pool_v = cache._planes[step.layer_id]
     out, lse = ops.paged_prefill(
         q, pool_k, pool_v, cache.page_table, step.batch_idx,
         block_mask.row_limit(step.input_pos, step.layer_id), cache.page_size, scale=scale, sinks=sinks,

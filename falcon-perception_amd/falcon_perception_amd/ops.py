@@ -19,14 +19,16 @@ def _rows(t: Tensor) -> Tensor:
 
 
 def kv_append(pool_k: Tensor, pool_v: Tensor, k: Tensor, v: Tensor, page_table: Tensor,
-              batch_idx: Tensor, input_pos: Tensor, page_size: int, clamp_negative: bool) -> None:
+              batch_idx: Tensor, input_pos: Tensor, page_size: int, clamp_negative: bool,
+              packed: bool = False) -> None:
     """Scatter k, v [T, H, S, D] into pool_k, pool_v [H, N, D] at the slots the page table gives.
 
     batch_idx [T] int64, input_pos [T, S] int32/int64.  Byte-exact copy
     (reference paged_attention.py:212-230 with clamp, :387-391 without).
+    `packed`: k, v are the prefill layout [1, H, L, D] with batch_idx, input_pos [1, L]; they are read as
+    L row groups of one token each through their strides.
     """
     N.require_cuda(pool_k, pool_v, k, v, page_table, batch_idx, input_pos)
-    T, H, S, D = k.shape
     if v.shape != k.shape:
         raise RuntimeError(f"k {tuple(k.shape)} and v {tuple(v.shape)} must have the same shape")
     if pool_k.dtype != k.dtype or pool_v.dtype != v.dtype:
@@ -34,20 +36,29 @@ def kv_append(pool_k: Tensor, pool_v: Tensor, k: Tensor, v: Tensor, page_table: 
     if not (pool_k.is_contiguous() and pool_v.is_contiguous()):
         raise RuntimeError("pool planes must be contiguous [H, N, D]")
     k, v = _rows(k), _rows(v)
-    input_pos = input_pos.contiguous()
-    batch_idx = batch_idx.contiguous()
+    if packed:
+        one, H, T, D = k.shape
+        S = 1
+        if one != 1 or batch_idx.numel() != T or input_pos.numel() != T:
+            raise RuntimeError("packed rows are [1, H, L, D] with L entries of batch_idx and input_pos")
+        ks, vs = (k.stride(2), k.stride(1), 0), (v.stride(2), v.stride(1), 0)
+    else:
+        T, H, S, D = k.shape
+        ks, vs = (k.stride(0), k.stride(1), k.stride(2)), (v.stride(0), v.stride(1), v.stride(2))
+    if not input_pos.is_contiguous():
+        input_pos = input_pos.contiguous()
+    if not batch_idx.is_contiguous():
+        batch_idx = batch_idx.contiguous()
     if batch_idx.dtype != torch.int64:
         batch_idx = batch_idx.to(torch.int64)
     if page_table.dtype != torch.int64 or page_table.stride(1) != 1:
         raise RuntimeError("page_table must be int64 with a dense last axis")
-    Hp, n_slots, Dp = pool_k.shape
     rc = N.lib().fp_kv_append(
-        pool_k.data_ptr(), pool_v.data_ptr(), k.data_ptr(), v.data_ptr(),
-        k.stride(0), k.stride(1), k.stride(2), v.stride(0), v.stride(1), v.stride(2),
+        pool_k.data_ptr(), pool_v.data_ptr(), k.data_ptr(), v.data_ptr(), *ks, *vs,
         page_table.data_ptr(), page_table.stride(0), batch_idx.data_ptr(),
         input_pos.data_ptr(), N.index_code(input_pos),
         T, H, S, D, page_size, page_table.shape[1], page_table.shape[0],
-        n_slots, N.dtype_code(k.dtype), int(clamp_negative), N.stream_ptr(k.device))
+        pool_k.shape[1], N.dtype_code(k.dtype), int(clamp_negative), N.stream_ptr(k.device))
     N.check(rc, "fp_kv_append")
 
 
@@ -328,11 +339,13 @@ def paged_prefill(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor,
     if Dp != D or pool_k.dtype != q.dtype or pool_v.dtype != q.dtype:
         raise RuntimeError("q / pool shape or dtype mismatch")
     q = _rows(q)
-    batch_idx = batch_idx.reshape(-1).contiguous()
-    row_limit = row_limit.reshape(-1).contiguous()
+    if not batch_idx.is_contiguous():
+        batch_idx = batch_idx.contiguous()
+    if not row_limit.is_contiguous():
+        row_limit = row_limit.contiguous()
     if batch_idx.dtype != torch.int64 or row_limit.dtype != torch.int32:
         raise RuntimeError("batch_idx must be int64 and row_limit int32")
-    if batch_idx.shape[0] != Lq or row_limit.shape[0] != Lq:
+    if batch_idx.numel() != Lq or row_limit.numel() != Lq:
         raise RuntimeError("batch_idx and row_limit need one entry per query row")
     if scale is None:
         scale = 1.0 / math.sqrt(D)

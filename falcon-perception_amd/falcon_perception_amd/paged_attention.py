@@ -78,6 +78,10 @@ class PagedKVCache(KVCacheBase):
 
         self.kv_shape = (num_layers, 2, 1, n_heads, n_pages * page_size, head_dim)
         self.kv_cache = torch.zeros(self.kv_shape, dtype=dtype, device=device)
+        # views of every layer's K and V planes, made once: [H, N, D] for the kernels, [1, H, N, D] as returned
+        # to the model (an indexing operation per layer and call costs the host more than the launch itself)
+        self._planes = [(self.kv_cache[l, 0, 0], self.kv_cache[l, 1, 0]) for l in range(num_layers)]
+        self._pools = [(self.kv_cache[l, 0], self.kv_cache[l, 1]) for l in range(num_layers)]
 
         # 1, or n_heads // n_kv_heads when the cached V heads are plain copies inside a group (the model's
         # repeat_kv, model.py:112-113): the decode kernel then reads V once per group.  Taken from the class
@@ -91,6 +95,7 @@ class PagedKVCache(KVCacheBase):
         self._workspace: Tensor | None = None
         self._decode_launch: dict[tuple, tuple[int, int]] = {}
         self._prefill_workspace: Tensor | None = None
+        self._prefill_need: dict[tuple, int] = {}
 
     # ------------------------------------------------------------------ append
     def insert_kv(self, layer_id: int, k: Tensor, v: Tensor, input_pos: Tensor | None = None,
@@ -115,10 +120,11 @@ class PagedKVCache(KVCacheBase):
         assert D_cache == K_D, "hidden dim must match"
         assert input_pos.shape == (B, S), "input_pos must have the same shape as val"
         assert batch_idx.shape == (B,), "batch_idx must have one dimension only"
-        ops.kv_append(self.kv_cache[layer_id, 0, 0], self.kv_cache[layer_id, 1, 0], k_val, v_val,
-                      self.page_table, batch_idx, input_pos, self.page_size, clamp_negative=True)
+        pool_k, pool_v = self._planes[layer_id]
+        ops.kv_append(pool_k, pool_v, k_val, v_val, self.page_table, batch_idx, input_pos, self.page_size,
+                      clamp_negative=True)
         self.last_decode_step = StepMeta(layer_id, input_pos, batch_idx)
-        return self.kv_cache[layer_id, 0], self.kv_cache[layer_id, 1]
+        return self._pools[layer_id]
 
     def assign_prefill_no_paging(self, layer_id: int, k_val: Tensor, v_val: Tensor, input_pos: Tensor,
                                  batch_idx: Tensor):
@@ -130,13 +136,10 @@ class PagedKVCache(KVCacheBase):
         assert input_pos.ndim == 2, "input_pos must be a 2D tensor"
         assert k_val.ndim == 4, "k_val must be a 4D tensor"
         assert v_val.ndim == 4, "v_val must be a 4D tensor"
-        L = batch_idx.shape[1]
-        # [1, H, L, D] seen as L row groups of one token each
-        k_rows = k_val[0].transpose(0, 1).unsqueeze(2)
-        v_rows = v_val[0].transpose(0, 1).unsqueeze(2)
-        ops.kv_append(self.kv_cache[layer_id, 0, 0], self.kv_cache[layer_id, 1, 0], k_rows, v_rows,
-                      self.page_table, batch_idx.reshape(L), input_pos.reshape(L, 1), self.page_size,
-                      clamp_negative=False)
+        pool_k, pool_v = self._planes[layer_id]
+        # [1, H, L, D] seen as L row groups of one token each: the strides say so, no views are made
+        ops.kv_append(pool_k, pool_v, k_val, v_val, self.page_table, batch_idx, input_pos, self.page_size,
+                      clamp_negative=False, packed=True)
         self.last_prefill_step = StepMeta(layer_id, input_pos, batch_idx)
         return k_val, v_val
 
@@ -158,14 +161,13 @@ class PagedKVCache(KVCacheBase):
             assert S == 1 and batch_idx.shape == (B,), "a decode step has one token per sequence"
         else:
             assert B == 1 and batch_idx.shape == (1, S), "a prefill step is one packed row"
-        q = ops.qkv_norm_rope_append(xq, xk, xv, freqs_cis, freqs_cis_2d, self.kv_cache[layer_id, 0, 0],
-                                     self.kv_cache[layer_id, 1, 0], self.page_table, batch_idx, input_pos,
-                                     self.page_size, clamp_negative=decode)
+        q = ops.qkv_norm_rope_append(xq, xk, xv, freqs_cis, freqs_cis_2d, *self._planes[layer_id], self.page_table,
+                                     batch_idx, input_pos, self.page_size, clamp_negative=decode)
         if decode:
             self.last_decode_step = StepMeta(layer_id, input_pos, batch_idx)
         else:
             self.last_prefill_step = StepMeta(layer_id, input_pos, batch_idx)
-        return q, self.kv_cache[layer_id, 0], self.kv_cache[layer_id, 1]
+        return (q, *self._pools[layer_id])
 
     def v_copies_are_identical(self, layer_id: int = 0) -> bool:
         """Whether the V plane of a layer really holds `kv_rep` identical heads per group (bit for bit, over
@@ -354,7 +356,10 @@ class PagedKVCache(KVCacheBase):
     def prefill_workspace(self, Lq: int, Hq: int, D: int, Hc: int, dtype: torch.dtype):
         """Scratch with which the prefill kernel cuts a small launch along the keys as well, owned by the
         cache and grown on demand (prefill steps are not captured in graphs); False when the shape needs none."""
-        need = ops.prefill_workspace_bytes(Lq, Hq, Hc, D, dtype)
+        key = (Lq, Hq, Hc, D, dtype)
+        need = self._prefill_need.get(key)
+        if need is None:
+            need = self._prefill_need[key] = ops.prefill_workspace_bytes(Lq, Hq, Hc, D, dtype)
         if need == 0:
             return False
         if self._prefill_workspace is None or self._prefill_workspace.numel() < need:
