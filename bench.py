@@ -47,6 +47,8 @@ DECODE_WORKLOADS = {
     "cfg5": dict(seed=5, dtype="bf16", B=256, Hq=32, Hc=8, D=128, P=128, n_pages=None, prefix=4096, lo=256, hi=12288),
     # cfg2 at the head_dim of the reference's OCR and 300M variants (reference __init__.py:78-85)
     "cfg2d64": dict(seed=2, dtype="bf16", B=64, Hq=16, Hc=8, D=64, P=128, n_pages=4096, prefix=1024, lo=64, hi=3072),
+    # cfg2 in the reference's default dtype (reference server/config.py:38)
+    "cfg2f32": dict(seed=2, dtype="f32", B=64, Hq=16, Hc=8, D=128, P=128, n_pages=4096, prefix=1024, lo=64, hi=3072),
 }
 DTYPES = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
 
@@ -893,7 +895,7 @@ def main() -> int:
         torch.cuda.empty_cache()
         # every other BASELINE config, the expanded-head cache of the reference's engine, head_dim 64
         legs = {}
-        for name in ("cfg1", "cfg2x", "cfg2xs", "cfg2d64", "cfg4d", "cfg5"):
+        for name in ("cfg1", "cfg2x", "cfg2xs", "cfg2d64", "cfg2f32", "cfg4d", "cfg5"):
             if name != args.workload:
                 legs[name] = decode_leg(name, hbm_budget_gb=args.hbm_budget_gb if name == "cfg5" else None,
                                         cpu=(name == "cfg1" and not args.no_cpu_baseline))

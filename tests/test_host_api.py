@@ -287,7 +287,7 @@ def test_bench_reads_traffic_from_the_profiles_and_refuses_several_gpus():
     import bench
 
     # the decode workloads share one summary (a line per workload), the other kernels have a file each
-    for wl in ("cfg1", "cfg2", "cfg2x", "cfg2xs", "cfg2d64", "cfg4d", "cfg5"):
+    for wl in ("cfg1", "cfg2", "cfg2x", "cfg2xs", "cfg2d64", "cfg2f32", "cfg4d", "cfg5"):
         t = bench.profiled_traffic("paged_decode", wl)
         assert t is not None and t > 1e6, wl
     for kernel in ("kv_append", "kv_gather", "qkv_rope_append"):
