@@ -604,7 +604,7 @@ def small_batch_decode(steps: int = 200) -> dict:
     return out
 
 
-def decode_leg(name: str, steps: int = 20, hbm_budget_gb: float | None = None, cpu: bool = False) -> dict:
+def decode_leg(name: str, steps: int = 50, hbm_budget_gb: float | None = None, cpu: bool = False) -> dict:
     """One more decode workload next to the headline: the fused step (append inside the split-K pass + merge)
     timed like the headline, the split-K pass alone by events, both priced with the workload's algorithmic
     bytes."""
@@ -615,7 +615,7 @@ def decode_leg(name: str, steps: int = 20, hbm_budget_gb: float | None = None, c
             return {"skipped": f"only {free / 1e9:.0f} GB of HBM free: no room for a long-context pool"}
     case = make_decode_case(name, hbm_budget_gb=hbm_budget_gb)
     c = case.cfg
-    ms_step = time_steps(case.run_fused, steps, 5, samples=11)
+    ms_step = time_steps(case.run_fused, steps, 10)
     ms_partial = event_ms(lambda: case.attend("partial"), steps, batch=10)
     alg_decode, alg_append = case.bytes_decode(), case.bytes_append()
     gbps = (alg_decode + alg_append) / (ms_step * 1e-3) / 1e9
