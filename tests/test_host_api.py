@@ -297,3 +297,24 @@ def test_bench_reads_traffic_from_the_profiles_and_refuses_several_gpus():
     assert 666.0e6 < bench.profiled_traffic("paged_decode", "cfg2") < 1.05 * 666.1e6
     res = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert res.returncode == 2 and "ONE GPU" in res.stderr and not res.stdout.strip()
+
+
+def test_noalloc_entry_point_rejects_what_its_array_cannot_hold(native_lib):
+    # host-side checks only: nothing below reaches the GPU
+    args = lambda B, split: (None, 0, 0, None, None, None, 0, None, None, 0, None, 0, 0, None, None,
+                             B, 32, 32, 1, 128, 16, 512, 4, 128, 8192, split, 1.0, 1, None)
+    rc = native_lib.fp_paged_decode_noalloc(*args(4096, 64))
+    assert rc == -4 and b"the library's array holds" in native_lib.fp_last_error()
+    assert native_lib.fp_paged_decode_workspace_bytes(4096, 32, 128, 8192, 64) > _native.NOALLOC_SCRATCH_BYTES
+    assert native_lib.fp_paged_decode_noalloc(*args(-1, 64)) == -1
+    assert native_lib.fp_paged_decode_noalloc(*args(4, 100)) == -1 and b"multiple of 64" in native_lib.fp_last_error()
+    # the header's limit and the Python mirror agree
+    text = open(os.path.join(ROOT, "include", "fp_paged_kv.h")).read()
+    assert re.search(r"#define FP_NOALLOC_SCRATCH_BYTES \(64ll << 20\)", text) and _native.NOALLOC_SCRATCH_BYTES == 64 << 20
+
+
+def test_hybrid_row_limits_argument_errors(native_lib):
+    assert native_lib.fp_hybrid_row_limits(None, None, None, 0, -1, 1, 2, None, None, None) == -1
+    assert native_lib.fp_hybrid_row_limits(None, None, None, 0, 70000, 1, 2, None, None, None) == -2
+    assert native_lib.fp_hybrid_row_limits(None, None, None, 0, 0, 1, 2, None, None, None) == 0  # an empty row is fine
+    assert native_lib.fp_hybrid_row_limits(None, None, None, 0, 5, 1, 2, None, None, None) == -1  # null pointers
