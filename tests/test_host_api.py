@@ -37,6 +37,43 @@ def test_library_exports_every_declared_symbol(native_lib):
     assert native_lib.fp_abi_version() == _native.FP_ABI_VERSION
 
 
+def header_declarations():
+    """name -> number of parameters, from the C declarations of the header."""
+    text = open(os.path.join(ROOT, "include", "fp_paged_kv.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"//[^\n]*", "", text)
+    decls = {}
+    for name, params in re.findall(r"\b(fp_[a-z0-9_]+)\s*\(([^()]*)\)\s*;", text):
+        params = params.strip()
+        decls[name] = 0 if params in ("", "void") else params.count(",") + 1
+    return decls
+
+
+def test_ctypes_signatures_have_the_arity_of_the_header():
+    decls = header_declarations()
+    assert sorted(decls) == header_functions()
+    for name, n in decls.items():
+        restype, argtypes = _native.SIGNATURES[name]
+        assert len(argtypes) == n, f"{name}: header declares {n} parameters, the binding passes {len(argtypes)}"
+
+
+def test_header_is_plain_c(tmp_path):
+    """The boundary is a C ABI: the header must compile as C99 and as C++ with nothing but the standard headers."""
+    import shutil
+    import subprocess
+
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    names = header_functions()
+    src = tmp_path / "use_header.c"
+    table = ", ".join(f"(void (*)(void)){n}" for n in names)
+    src.write_text('#include "fp_paged_kv.h"\nvoid (*const fp_table[])(void) = {' + table + "};\n")
+    inc = os.path.join(ROOT, "include")
+    for cmd in (["gcc", "-std=c99", "-pedantic", "-Wall", "-Werror"], ["g++", "-x", "c++", "-std=c++11", "-Wall", "-Werror"]):
+        res = subprocess.run(cmd + ["-I", inc, "-fsyntax-only", str(src)], capture_output=True, text=True)
+        assert res.returncode == 0, res.stderr
+
+
 def test_argument_errors_come_back_as_codes_not_crashes(native_lib):
     # no device work: every call below is rejected by the host-side checks
     assert native_lib.fp_paged_decode_workspace_bytes(4, 8, 128, 1024, 100) < 0  # split not a multiple of 64
