@@ -48,7 +48,7 @@ def close(got, want, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=str)
-@pytest.mark.parametrize("D,Hq,Hkv", [(128, 4, 2), (64, 8, 8), (128, 6, 2)])
+@pytest.mark.parametrize("D,Hq,Hkv", [(128, 4, 2), (64, 8, 8), (128, 6, 2), (128, 8, 2), (64, 8, 1), (128, 16, 8)])
 def test_prefill_step(dtype, D, Hq, Hkv):
     P = 16
     st = PagedState(31, n_pages=64, page_size=P, max_batch=6, Hc=Hq, D=D, dtype=dtype)
