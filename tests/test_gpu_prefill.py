@@ -247,3 +247,21 @@ def test_span_open_across_a_document_boundary_is_refused():
         st.cache.create_prefill_blockmask(dev(bidx), dev(ids), SOI, EOI)
     # unchecked, the call returns as before (the mask of such a row is unspecified)
     st.cache.create_prefill_blockmask(dev(bidx), dev(ids), SOI, EOI, validate=False)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=str)
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("G", [1, 2, 4, 8])
+@pytest.mark.parametrize("P", [64, 16, 24], ids=["page-holds-tile", "small-page", "odd-page"])
+def test_every_kernel_instance(dtype, D, G, P):
+    """One small packed step per template instance (dtype, head_dim, query heads per cache head, and
+    the three ways a key tile is staged: whole tiles from a page, row by row with a power-of-two page, row by
+    row with any other page size): two sequences packed without padding, the second with an image span."""
+    layout = layout_for([(1, 70, 0, 0), (2, 9, 60, 45)])
+    ids, bidx, pos = repack(layout, 1)
+    st = PagedState(40 + G, n_pages=24, page_size=P, max_batch=4, Hc=1, D=D, dtype=dtype)
+    for slot in (1, 2):
+        st.add_sequence(int((bidx == slot).sum()))
+    q, k, v, out, lse = prefill_through_api(st, ids, bidx, pos, G, dtype, 1)
+    eo, el = O.prefill_attention_packed(f64(q), f64(k), f64(v), bidx[None], ids[None], SOI, EOI)
+    assert_close(out, lse, eo, el, dtype)
