@@ -394,3 +394,34 @@ def test_one_position_and_slot_per_sequence_is_required():
     q = randn(st.gen, (3, 1, 1, 64), torch.bfloat16)
     with pytest.raises(RuntimeError, match="one entry per sequence"):
         run_decode(st, q, torch.tensor([4, 8], dtype=torch.int32))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=str)
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("G", [1, 2, 4, 8])
+@pytest.mark.parametrize("P", [64, 24], ids=["aligned-pages", "odd-pages"])
+def test_every_instance_of_the_even_cut(dtype, D, G, P):
+    """One launch per template instance of the split-K pass in its even-cut form (4 cache heads x 96 sequences
+    x 8 splits = 3072 workgroups, more than the GPU holds at once), fused append included; where a workgroup
+    serves several query heads, also on the expanded cache (one cached head per query head, V copies
+    identical, read once per group)."""
+    B, Hc, split, ctx = 96, 4, 64, 512
+    lens = torch.randint(0, ctx - 1, (B,), generator=torch.Generator().manual_seed(70 + G)).tolist()
+    lens[0], lens[1], lens[2] = ctx - 1, 0, 64
+    for rep in (1, G) if G in (2, 4) else (1,):  # a group read as one is 2 or 4 heads wide
+        H_pool = Hc * rep
+        st = PagedState(60 + G, n_pages=B * (-(-ctx // P)) + 8, page_size=P, max_batch=B + 2, Hc=H_pool, D=D, dtype=dtype)
+        for L in lens:
+            st.add_sequence(L + 1)
+        st.lens = lens
+        st.prefill_random()
+        if rep > 1:  # make the V copies of a group identical, as repeat_kv leaves them
+            _, pv = st.pool_planes()
+            pv.copy_(pv.view(Hc, rep, *pv.shape[1:])[:, :1].expand(Hc, rep, *pv.shape[1:]).reshape(pv.shape).clone())
+        q = randn(st.gen, (B, Hc * G, 1, D), dtype)
+        k_new = randn(st.gen, (B, H_pool, 1, D), dtype).to(DEV)
+        v_new = randn(st.gen, (B, Hc, 1, D), dtype).repeat_interleave(rep, dim=1).to(DEV)
+        pos = torch.tensor(lens, dtype=torch.int32)
+        out, lse = run_decode(st, q, pos, k_new=k_new, v_new=v_new, split_tokens=split, max_context=ctx, kv_rep=rep)
+        eo, el = oracle_decode(st, q, pos)  # the pool now holds the new rows
+        assert_close(out, lse, eo, el, dtype)
