@@ -63,18 +63,21 @@ def test_cfg1_cpu_reference_shape_fp32():
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=str)
 @pytest.mark.parametrize("D", [64, 128])
 @pytest.mark.parametrize("G", [1, 2, 4, 8])
-def test_context_boundaries_and_gqa(dtype, D, G):
-    P = 16
-    st = PagedState(2, n_pages=80, page_size=P, max_batch=12, Hc=2, D=D, dtype=dtype)
+@pytest.mark.parametrize("P", [16, 128, 24])
+def test_context_boundaries_and_gqa(dtype, D, G, P):
+    """Contexts at every page and split boundary, for every template instance of the split-by-split pass:
+    one split that stores its result directly (split_tokens 512), several splits and the merge pass; page
+    sizes whose rows a load instruction covers exactly (128), smaller (16) and no power of two (24)."""
     lens = [1, 2, P - 1, P, P + 1, 4 * P, 4 * P + 1, 63, 64, 65, 300]
+    st = PagedState(2, n_pages=sum(-(-L // P) for L in lens) + 4, page_size=P, max_batch=12, Hc=2, D=D, dtype=dtype)
     for L in lens:
         st.add_sequence(L)
     st.prefill_random()
     q = randn(st.gen, (len(lens), 2 * G, 1, D), dtype)
     pos = torch.tensor([L - 1 for L in lens], dtype=torch.int32)
     eo, el = oracle_decode(st, q, pos)
-    for split in (0, 64, 128):
-        out, lse = run_decode(st, q, pos, split_tokens=split, max_context=320)
+    for split in (0, 64, 128, 512):
+        out, lse = run_decode(st, q, pos, split_tokens=split, max_context=max(lens) + 20)
         assert_close(out, lse, eo, el, dtype)
 
 
