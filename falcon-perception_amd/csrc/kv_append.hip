@@ -47,6 +47,7 @@ struct AppendArgs {
   int max_batch;
   int64_t n_slots;
   int clamp_negative;
+  int64_t item0;  // first item of this launch: a launch holds fewer than 2^32 lanes, a larger append is several
 };
 
 constexpr int kThreads = 256;
@@ -60,7 +61,7 @@ template <typename Vec, bool kTokenMajor, typename Idx>
 __global__ __launch_bounds__(kThreads) void kv_append_kernel(const AppendArgs a, int H) {
   const Idx per_tok = kTokenMajor ? static_cast<Idx>(H) * a.chunks : static_cast<Idx>(a.chunks);
   const Idx items = static_cast<Idx>(a.n_tok) * per_tok;
-  const Idx i = static_cast<Idx>(blockIdx.x) * kThreads + threadIdx.x;
+  const Idx i = static_cast<Idx>(a.item0) + static_cast<Idx>(blockIdx.x) * kThreads + threadIdx.x;
   if (i >= items) return;
   const int tok = static_cast<int>(i / per_tok);
   int c = static_cast<int>(i - static_cast<Idx>(tok) * per_tok);
@@ -96,25 +97,33 @@ __global__ __launch_bounds__(kThreads) void kv_append_kernel(const AppendArgs a,
   __builtin_nontemporal_store(vreg, reinterpret_cast<Vec*>(a.pool_v + dst));
 }
 
+// A dispatch holds fewer than 2^32 lanes in each grid dimension: a larger append goes out as several launches of
+// 2^31 lanes, each told where its items start.
+constexpr int64_t kLaunchBlocks = (1ll << 31) / kThreads;
+
 template <typename Vec>
-int launch(const AppendArgs& a, int H, hipStream_t stream) {
+int launch(const AppendArgs& a0, int H, hipStream_t stream) {
   // the source's memory order decides which index runs fastest across the lanes
-  const bool token_major = a.ks_h <= a.ks_t && a.vs_h <= a.vs_t;
-  const int64_t per_grid_row = static_cast<int64_t>(a.n_tok) * a.chunks * (token_major ? H : 1);
+  const bool token_major = a0.ks_h <= a0.ks_t && a0.vs_h <= a0.vs_t;
+  const int64_t per_grid_row = static_cast<int64_t>(a0.n_tok) * a0.chunks * (token_major ? H : 1);
   const int64_t blocks = (per_grid_row + kThreads - 1) / kThreads;
-  if (blocks > INT32_MAX) return fp::fail(FP_ERR_UNSUPPORTED, "fp_kv_append: more than 2^31-1 workgroups");
   const bool narrow = per_grid_row + kThreads < (1ll << 32);
-  dim3 grid(static_cast<unsigned>(blocks), token_major ? 1u : static_cast<unsigned>(H));
-  if (token_major) {
-    if (narrow)
-      hipLaunchKernelGGL((kv_append_kernel<Vec, true, uint32_t>), grid, dim3(kThreads), 0, stream, a, H);
-    else
-      hipLaunchKernelGGL((kv_append_kernel<Vec, true, int64_t>), grid, dim3(kThreads), 0, stream, a, H);
-  } else {
-    if (narrow)
-      hipLaunchKernelGGL((kv_append_kernel<Vec, false, uint32_t>), grid, dim3(kThreads), 0, stream, a, H);
-    else
-      hipLaunchKernelGGL((kv_append_kernel<Vec, false, int64_t>), grid, dim3(kThreads), 0, stream, a, H);
+  AppendArgs a = a0;
+  for (int64_t b0 = 0; b0 < blocks; b0 += kLaunchBlocks) {
+    a.item0 = b0 * kThreads;
+    const int64_t nb = blocks - b0 < kLaunchBlocks ? blocks - b0 : kLaunchBlocks;
+    dim3 grid(static_cast<unsigned>(nb), token_major ? 1u : static_cast<unsigned>(H));
+    if (token_major) {
+      if (narrow)
+        hipLaunchKernelGGL((kv_append_kernel<Vec, true, uint32_t>), grid, dim3(kThreads), 0, stream, a, H);
+      else
+        hipLaunchKernelGGL((kv_append_kernel<Vec, true, int64_t>), grid, dim3(kThreads), 0, stream, a, H);
+    } else {
+      if (narrow)
+        hipLaunchKernelGGL((kv_append_kernel<Vec, false, uint32_t>), grid, dim3(kThreads), 0, stream, a, H);
+      else
+        hipLaunchKernelGGL((kv_append_kernel<Vec, false, int64_t>), grid, dim3(kThreads), 0, stream, a, H);
+    }
   }
   return FP_OK;
 }
@@ -150,7 +159,7 @@ extern "C" int fp_kv_append(void* pool_k, void* pool_v, const void* k, const voi
                v_stride_t * eb, v_stride_h * eb, v_stride_s * eb,
                page_table, pt_row_stride, batch_idx, input_pos,
                pos_index_type == FP_INDEX_I64, T * S, S, 0, D * eb, fp::PageDiv(page_size),
-               n_pages, max_batch, n_slots, clamp_negative};
+               n_pages, max_batch, n_slots, clamp_negative, 0};
 
   // widest vector every row address is a multiple of
   int vec = 16;

@@ -34,6 +34,7 @@ struct GatherArgs {
   int n_pages;
   int max_batch;
   int64_t n_slots;
+  int64_t item0;  // first item of this launch: a launch holds fewer than 2^32 lanes in x, a longer gather is several
 };
 
 constexpr int kThreads = 256;
@@ -44,7 +45,7 @@ __global__ __launch_bounds__(kThreads) void kv_gather_kernel(const GatherArgs a)
   const int h = blockIdx.y;
   const int b = blockIdx.z;
   const int64_t items = static_cast<int64_t>(a.max_len) * a.chunks;
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  const int64_t i = a.item0 + static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (i >= items) return;
 
   int64_t len = fp::load_index(a.seq_lens, b, a.len_i64);
@@ -73,12 +74,19 @@ __global__ __launch_bounds__(kThreads) void kv_gather_kernel(const GatherArgs a)
   __builtin_nontemporal_store(reg, reinterpret_cast<Vec*>(a.out + dst));
 }
 
+constexpr int64_t kLaunchBlocks = (1ll << 31) / kThreads;  // a dispatch holds fewer than 2^32 lanes in x
+
 template <typename Vec>
-void launch_gather(const GatherArgs& a, int B, int H, hipStream_t stream) {
-  const int64_t items = static_cast<int64_t>(a.max_len) * a.chunks;
-  dim3 grid(static_cast<unsigned>((items + kThreads - 1) / kThreads), static_cast<unsigned>(H),
-            static_cast<unsigned>(B));
-  hipLaunchKernelGGL(kv_gather_kernel<Vec>, grid, dim3(kThreads), 0, stream, a);
+void launch_gather(const GatherArgs& a0, int B, int H, hipStream_t stream) {
+  const int64_t items = static_cast<int64_t>(a0.max_len) * a0.chunks;
+  const int64_t blocks = (items + kThreads - 1) / kThreads;
+  GatherArgs a = a0;
+  for (int64_t b0 = 0; b0 < blocks; b0 += kLaunchBlocks) {
+    a.item0 = b0 * kThreads;
+    const int64_t nb = blocks - b0 < kLaunchBlocks ? blocks - b0 : kLaunchBlocks;
+    dim3 grid(static_cast<unsigned>(nb), static_cast<unsigned>(H), static_cast<unsigned>(B));
+    hipLaunchKernelGGL(kv_gather_kernel<Vec>, grid, dim3(kThreads), 0, stream, a);
+  }
 }
 
 __global__ __launch_bounds__(kThreads) void convert_block_ids_kernel(
@@ -123,7 +131,7 @@ extern "C" int fp_kv_gather(const void* pool, void* out, int64_t out_stride_b, i
   GatherArgs a{static_cast<const char*>(pool), static_cast<char*>(out),
                out_stride_b * eb, out_stride_h * eb, out_stride_t * eb,
                page_table, pt_row_stride, batch_idx, seq_lens, len_index_type == FP_INDEX_I64,
-               max_len, 0, D * eb, fp::PageDiv(page_size), n_pages, max_batch, n_slots};
+               max_len, 0, D * eb, fp::PageDiv(page_size), n_pages, max_batch, n_slots, 0};
   int vec = 16;
   auto fits = [&](int n) {
     return a.row_bytes % n == 0 && a.os_b % n == 0 && a.os_h % n == 0 && a.os_t % n == 0 &&

@@ -418,8 +418,10 @@ extern "C" int fp_qkv_norm_rope_append(const void* xq, const void* xk, const voi
       !fp::aligned(pool_k, 16) || !fp::aligned(pool_v, 16) || !fp::aligned(freqs_cis, 8) ||
       (freqs_cis_2d && !fp::aligned(freqs_cis_2d, 8)))
     return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_qkv_norm_rope_append: rows must be 16-byte aligned");
-  if (static_cast<int64_t>(T) * (Hq + 2 * Hkv) / (kThreads / tpr) + 1 > INT32_MAX)
-    return fp::fail(FP_ERR_UNSUPPORTED, "fp_qkv_norm_rope_append: too many rows");
+  // a dispatch holds fewer than 2^32 lanes
+  if ((static_cast<int64_t>(T) * (Hq + 2 * Hkv) + kThreads) * tpr >= (1ll << 32))
+    return fp::fail(FP_ERR_UNSUPPORTED, "fp_qkv_norm_rope_append: too many rows for one launch (%lld lanes)",
+                    static_cast<long long>(T) * (Hq + 2 * Hkv) * tpr);
 
   RopeArgs a{static_cast<const char*>(xq), static_cast<const char*>(xk), static_cast<const char*>(xv),
              q_stride_t * eb, q_stride_h * eb, k_stride_t * eb, k_stride_h * eb, v_stride_t * eb, v_stride_h * eb,

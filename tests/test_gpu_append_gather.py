@@ -220,3 +220,34 @@ def test_large_append_round_trip_and_checksum():
     # nothing else was written: the pool holds exactly the appended rows (sum of bit patterns)
     assert int(pk.view(torch.int16).to(torch.int64).sum()) == int(k.view(torch.int16).to(torch.int64).sum())
     assert int(pv.view(torch.int16).to(torch.int64).sum()) == int(v.view(torch.int16).to(torch.int64).sum())
+
+
+def test_append_and_gather_with_more_than_2_32_vectors_in_a_launch():
+    """Rows of 3 bf16 values move as 2-byte vectors, one per lane; 1 435 000 000 such rows are more than
+    2^32 lanes in one launch, the case in which the kernels index their lanes with 64 bits.  One sequence
+    whose pages lie in reverse order; checked on the GPU (the pool, read back page by page, is the
+    input, and the gather returns it), bit for bit."""
+    free, _ = torch.cuda.mem_get_info()
+    assert free > 90e9, f"only {free / 1e9:.0f} GB of HBM free: this case holds about 60 GB"
+    S, D, P = 1_435_000_000, 3, 128
+    assert S * D > 2**32
+    n_pages = -(-S // P)
+    n_slots = n_pages * P
+    g = torch.Generator(device=DEV).manual_seed(11)
+    k = torch.randint(-32768, 32767, (1, 1, S, D), generator=g, device=DEV, dtype=torch.int16).view(torch.bfloat16)
+    v = torch.randint(-32768, 32767, (1, 1, S, D), generator=g, device=DEV, dtype=torch.int16).view(torch.bfloat16)
+    pool_k = torch.zeros((1, n_slots, D), dtype=torch.bfloat16, device=DEV)
+    pool_v = torch.zeros((1, n_slots, D), dtype=torch.bfloat16, device=DEV)
+    page_table = torch.zeros((2, n_pages), dtype=torch.int64, device=DEV)
+    page_table[1] = torch.arange(n_pages - 1, -1, -1, device=DEV)
+    bidx = torch.ones(1, dtype=torch.int64, device=DEV)
+    pos = torch.arange(S, dtype=torch.int32, device=DEV)[None]
+    ops.kv_append(pool_k, pool_v, k, v, page_table, bidx, pos, P, clamp_negative=False)
+    del pos
+    for pool, src in ((pool_k, k), (pool_v, v)):
+        back = pool.view(n_pages, P, D).flip(0).reshape(n_slots, D)[:S]
+        assert torch.equal(back.view(torch.int16), src[0, 0].view(torch.int16))
+        del back
+    lens = torch.tensor([S], dtype=torch.int64, device=DEV)
+    got = ops.kv_gather(pool_k, page_table, bidx, lens, P, S)
+    assert torch.equal(got[0, 0].view(torch.int16), k[0, 0].view(torch.int16))
