@@ -50,6 +50,18 @@ def close(got, want, dtype):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=str)
 @pytest.mark.parametrize("D,Hq,Hkv", [(128, 4, 2), (64, 8, 8), (128, 6, 2), (128, 8, 2), (64, 8, 1), (128, 16, 8)])
 def test_prefill_step(dtype, D, Hq, Hkv):
+    prefill_step(dtype, D, Hq, Hkv)
+
+
+@pytest.mark.parametrize("dtype,D,Hq,Hkv", [(torch.bfloat16, 32, 4, 2), (torch.bfloat16, 256, 4, 2), (torch.bfloat16, 512, 2, 1),
+                                            (torch.float32, 16, 4, 2), (torch.float32, 256, 2, 2), (torch.float16, 32, 2, 2),
+                                            (torch.float16, 256, 3, 1)], ids=str)
+def test_prefill_step_at_other_head_dims(dtype, D, Hq, Hkv):
+    """Rows of 4 to 64 sixteen-byte vectors: every lane-group width of the two kernels."""
+    prefill_step(dtype, D, Hq, Hkv)
+
+
+def prefill_step(dtype, D, Hq, Hkv):
     P = 16
     st = PagedState(31, n_pages=64, page_size=P, max_batch=6, Hc=Hq, D=D, dtype=dtype)
     lens = [37, 150, 64]
