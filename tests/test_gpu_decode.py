@@ -428,3 +428,46 @@ def test_every_instance_of_the_even_cut(dtype, D, G, P):
         out, lse = run_decode(st, q, pos, k_new=k_new, v_new=v_new, split_tokens=split, max_context=ctx, kv_rep=rep)
         eo, el = oracle_decode(st, q, pos)  # the pool now holds the new rows
         assert_close(out, lse, eo, el, dtype)
+
+
+@pytest.mark.parametrize("B", [1024, 1025, 3000])
+def test_more_sequences_than_the_even_cut_keeps_in_lds(B):
+    """The even cut holds the lengths of at most 1024 sequences; one more and the launch goes split by split
+    (9000 and more workgroups).  Short contexts, some empty, fused append."""
+    dtype, P, D, Hc, G = torch.bfloat16, 16, 64, 2, 2
+    gen = torch.Generator().manual_seed(B)
+    lens = torch.randint(0, 200, (B,), generator=gen).tolist()
+    lens[3], lens[B - 1] = 0, 199
+    st = PagedState(B, n_pages=sum(-(-(L + 1) // P) for L in lens) + 4, page_size=P, max_batch=B + 2, Hc=Hc, D=D, dtype=dtype)
+    for L in lens:
+        st.add_sequence(L + 1)
+    st.lens = lens
+    st.prefill_random()
+    q = randn(st.gen, (B, Hc * G, 1, D), dtype)
+    k_new, v_new = randn(st.gen, (B, Hc, 1, D), dtype).to(DEV), randn(st.gen, (B, Hc, 1, D), dtype).to(DEV)
+    pos = torch.tensor(lens, dtype=torch.int32)
+    out, lse = run_decode(st, q, pos, k_new=k_new, v_new=v_new, split_tokens=64, max_context=256)
+    eo, el = oracle_decode(st, q, pos)
+    assert_close(out, lse, eo, el, dtype)
+
+
+@pytest.mark.parametrize("P", [128, 16])
+def test_one_sequence_of_a_million_tokens(P):
+    """Context 1 000 000 on one cache head: thousands of splits (or long even-cut chunks with more page ids
+    than a workgroup keeps), positions near 2^20; against the float64 oracle."""
+    dtype, D, ctx = torch.bfloat16, 128, 1_000_000
+    st = PagedState(5, n_pages=-(-(ctx + 1) // P) + 3, page_size=P, max_batch=3, Hc=1, D=D, dtype=dtype)
+    st.add_sequence(ctx)
+    pk, pv = st.pool_planes()
+    g = torch.Generator(device=DEV).manual_seed(5)
+    pk.copy_(torch.randn(pk.shape, generator=g, device=DEV, dtype=torch.float32))
+    pv.copy_(torch.randn(pv.shape, generator=g, device=DEV, dtype=torch.float32))
+    q = randn(st.gen, (1, 2, 1, D), dtype)
+    pos = torch.tensor([ctx - 1], dtype=torch.int32)
+    eo, el = oracle_decode(st, q, pos)
+    for split in (0, 256, 65536 if P == 128 else 8192):
+        out, lse = run_decode(st, q, pos, split_tokens=split, max_context=ctx)
+        assert_close(out, lse, eo, el, dtype)
+    if P == 16:  # a split holds the ids of at most 1022 pages: a wider one is refused, not truncated
+        with pytest.raises(RuntimeError, match="spans more than"):
+            run_decode(st, q, pos, split_tokens=65536, max_context=ctx)
