@@ -235,6 +235,12 @@ PREFILL_WORKLOADS = {
     "cfg3x": dict(seed=3, dtype="bf16", n_seq=8, Hq=16, Hc=16, D=128, P=128, prefix_lo=256, prefix_hi=4096, chunk=512),
     # cfg3 at the head_dim of the OCR and 300M variants
     "cfg3d64": dict(seed=3, dtype="bf16", n_seq=8, Hq=16, Hc=8, D=64, P=128, prefix_lo=256, prefix_hi=4096, chunk=512),
+    # whole sequences as the reference's engine prefills them (paged_inference.py:637-672): on its cache of one head per
+    # query head, and at head_dim 64
+    "cfg3wx": dict(seed=3, dtype="bf16", n_seq=8, Hq=16, Hc=16, D=128, P=128, prefix_lo=256, prefix_hi=4096, chunk=512,
+                   whole=True),
+    "cfg3wd64": dict(seed=3, dtype="bf16", n_seq=8, Hq=16, Hc=8, D=64, P=128, prefix_lo=256, prefix_hi=4096, chunk=512,
+                     whole=True),
 }
 
 
@@ -573,6 +579,8 @@ def prefill_rate(steps: int = 10, name: str = "cfg3") -> dict:
     what = {"cfg3": "cfg3: 8 sequences, paged prefix U[256,4096], 512-token chunk each, 16 q / 8 kv heads, D 128",
             "cfg3w": "cfg3w: the same 8 sequences prefilled whole (prefix + chunk rows in one step, prefix rows see "
                      "their whole image span), 16 q / 8 kv heads, D 128",
+            "cfg3wx": "cfg3w on the reference engine's cache: one cached head per query head (16 q / 16 cached heads)",
+            "cfg3wd64": "cfg3w at head_dim 64",
             "cfg3f32": "cfg3 in fp32",
             "cfg3x": "cfg3 on the reference engine's cache: one cached head per query head (16 q / 16 cached heads)",
             "cfg3d64": "cfg3 at head_dim 64 (the reference's OCR and 300M variants)",
@@ -907,6 +915,9 @@ def main() -> int:
         result["chunked_prefill_head_dim_64"] = prefill_rate(name="cfg3d64")
         result["chunked_prefill_fp32"] = prefill_rate(name="cfg3f32")
         result["chunked_prefill_one_sequence"] = prefill_rate(name="cfg3one")
+        result["prefill_whole_sequences"] = prefill_rate(name="cfg3w")
+        result["prefill_whole_sequences_expanded_heads"] = prefill_rate(name="cfg3wx")
+        result["prefill_whole_sequences_head_dim_64"] = prefill_rate(name="cfg3wd64")
         result["decode_small_batch"] = small_batch_decode()
     print(json.dumps(result))
     return 0
