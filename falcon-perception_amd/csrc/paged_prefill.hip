@@ -9,7 +9,8 @@
 // sequence are visible.
 //
 // MFMA-bound.  A workgroup of 8 wavefronts owns one cache head and 256 / G consecutive packed
-// query rows of each of its G query heads; a wavefront owns 32 rows of one query head.
+// query rows of each of its G query heads; a wavefront owns 32 rows of one query head.  (Large launches
+// at head_dim 64 use workgroups of 4 wavefronts and 128 / G rows, two to a CU.)
 //   S^T = K Q^T  (v_mfma_f32_32x32x16): keys are the M rows, queries the N columns, so a
 //         lane holds scores of ONE query and softmax row reductions stay in registers
 //         (plus one exchange between the two lane halves).
@@ -147,17 +148,18 @@ struct Swizzle {
 // 32 query rows: every head of the group works from the same staged K/V tile, so the bytes that
 // travel from L2 into LDS (64 B per cycle and CU, and a wavefront waits at its load instructions
 // while that path is busy) are shared by all of them.
-template <typename E, int D, int G, bool kPow2>
-__global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const PrefillArgs a) {
+template <typename E, int D, int G, bool kPow2, int W = kWaves>
+__global__ __launch_bounds__(W * 64, 2) void paged_prefill_kernel(const PrefillArgs a) {
+  constexpr int kThreads = W * 64;  // shadows the file-scope constant: W wavefronts per workgroup
   using SW = Swizzle<D>;
   constexpr int MB = 1;                    // 32-row blocks per wavefront
-  constexpr int RB = kWaves / G;           // 32-row blocks per workgroup
+  constexpr int RB = W / G;                // 32-row blocks per workgroup
   constexpr int BM = RB * 32;              // query rows per workgroup
   constexpr int ROWB = D * 2;              // bytes of a K/V row
   constexpr int CPR = SW::CPR;
   constexpr int R32 = SW::R32;
   constexpr int RPI = 64 / CPR;            // rows one wavefront load instruction brings in
-  constexpr int NI = kTileN / (RPI * kWaves);  // load instructions per wavefront, tile and tensor
+  constexpr int NI = kTileN / (RPI * W);   // load instructions per wavefront, tile and tensor
   constexpr int DS = D / 16;               // MFMA k-steps over head_dim
   constexpr int DB = D / 32;               // 32-wide blocks of head_dim in O^T
   constexpr int TILE_BYTES = kTileN * ROWB;
@@ -169,7 +171,7 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
   __shared__ __attribute__((aligned(1024))) char s_v0[TILE_BYTES];
   __shared__ __attribute__((aligned(1024))) char s_v1[TILE_BYTES];
   __shared__ int s_bidx[BM];
-  __shared__ int s_red[kWaves];
+  __shared__ int s_red[W];
   __shared__ int s_tslot[kSlotTable];
 
   // linear id = cache head + Hc * tile: all tiles that read one cache head run on the XCD that
@@ -222,11 +224,11 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
   const char* vplane = a.pool_v + static_cast<int64_t>(hc) * a.n_slots * ROWB;
 
   // ---- per-lane constants of the staging loads and of the operand reads ----
-  // load instruction i of this wavefront fills LDS rows (i * kWaves + wave) * RPI .. + RPI; this lane
+  // load instruction i of this wavefront fills LDS rows (i * W + wave) * RPI .. + RPI; this lane
   // fills position lp of row lrow in that group.  kswz / vrot of the row do not depend on i.
   const int lrow = lane / CPR;
   const int lp = lane % CPR;
-  const int st_row0 = wave * RPI + lrow;  // row of load instruction 0; instruction i adds i * kWaves * RPI
+  const int st_row0 = wave * RPI + lrow;  // row of load instruction 0; instruction i adds i * W * RPI
   const int k_src_off = (lp ^ SW::kswz(st_row0)) * 16;
   const int v_src_off = ((((lp >> 1) + R32 - SW::vrot(st_row0)) % R32) * 2 + (lp & 1)) * 16;
   // K operand: row kb * 32 + ln, chunk 2 * ds + half at position (2 * ds) ^ ksel
@@ -303,7 +305,7 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
     __syncthreads();
     int kv_max = 0;
 #pragma unroll
-    for (int w = 0; w < kWaves; ++w) kv_max = max(kv_max, s_red[w]);
+    for (int w = 0; w < W; ++w) kv_max = max(kv_max, s_red[w]);
     kv_max = __builtin_amdgcn_readfirstlane(kv_max);
     const int n_run_tiles = (kv_max + kTileN - 1) / kTileN;
     // this workgroup's share of the run's key tiles: [kt_lo, n_kv_tiles)
@@ -364,8 +366,8 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
     uint32_t lane_k[NI], lane_v[NI];  // byte offset of this lane's 16 bytes from the first row of a tile
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
-      lane_k[i] = (i * kWaves * RPI + st_row0) * ROWB + k_src_off;
-      lane_v[i] = (i * kWaves * RPI + st_row0) * ROWB + v_src_off;
+      lane_k[i] = (i * W * RPI + st_row0) * ROWB + k_src_off;
+      lane_v[i] = (i * W * RPI + st_row0) * ROWB + v_src_off;
     }
     // One staging load of tile kt, whose first slot is ts (or -1): pieces 0 .. NI - 1 are the V loads
     // of the row groups, NI .. 2 NI - 1 the K loads.  Tiles past the run's last one are not staged.
@@ -373,12 +375,12 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
       if (kt >= n_kv_tiles) return;
       const int i = piece % NI;
       const bool is_k = piece >= NI;
-      char* lds = dst + (i * kWaves + wave) * RPI * ROWB;  // wavefront-uniform
+      char* lds = dst + (i * W + wave) * RPI * ROWB;  // wavefront-uniform
       if (ts >= 0) {
         load_to_lds((is_k ? kplane : vplane) + static_cast<int64_t>(ts) * ROWB, is_k ? lane_k[i] : lane_v[i], lds);
       } else {
         asm volatile("");  // rare: keep it out of the way as a branch
-        const int kpos = kt * kTileN + i * kWaves * RPI + st_row0;
+        const int kpos = kt * kTileN + i * W * RPI + st_row0;
         int blkid, off;
         key_block(kpos, blkid, off);
         const bool in_range = kpos < kv_max && blkid < a.n_pages;
@@ -591,7 +593,7 @@ __global__ __launch_bounds__(kThreads, 2) void paged_prefill_kernel(const Prefil
     };
 
     // steps 0 .. n_my (the last one only has the O^T part of the last tile)
-    if (wave < kWaves / 2) {
+    if (wave < W / 2) {
       for (int i = 0; i <= n_my; i += 2) {
         step(IntC<0>{}, IntC<0>{}, i);
         if (i + 1 <= n_my) step(IntC<0>{}, IntC<1>{}, i + 1);
@@ -713,6 +715,7 @@ __global__ __launch_bounds__(kMergeRows * 64) void paged_prefill_merge_kernel(co
 }
 
 constexpr int kMaxKeyShares = 8;
+constexpr int kSmallWorkgroupsFrom = 1;  // eight-wavefront workgroups per CU from which a head_dim 64 launch uses four-wavefront ones
 
 // Key shares for a launch of `wgs` workgroups.  bf16 / f16: a launch that would leave at least half of the
 // CUs idle is cut along the keys until every CU has a workgroup.  (With about one workgroup per CU
@@ -742,6 +745,24 @@ void launch_group(const PrefillArgs& a0, void* workspace, int64_t workspace_byte
   if (shares > 1) {
     a.ws_ml = static_cast<float*>(workspace);
     a.ws_acc = reinterpret_cast<short*>(a.ws_ml + static_cast<int64_t>(shares) * a.Lq * a.Hq * 2);
+  }
+  // head_dim 64: a launch with at least one eight-wavefront workgroup per CU goes out as workgroups of four
+  // wavefronts, two to a CU.  A staged K/V tile then serves half as many query rows, but at 128-byte rows the
+  // staging is cheap, the softmax (which does not shrink with head_dim) is what a step waits for, and two
+  // independent workgroups per CU fill each other's barrier and set-up gaps: 8 x 512-row chunks 85 us against
+  // 91 us, the same 8 sequences whole 350 us against 370 us.  At head_dim 128 the same split is slower
+  // (whole sequences 564 us against 485 us): the staging path is the limit there.
+  if constexpr (G <= 4 && D == 64) {
+    if (shares == 1 && static_cast<int64_t>(a.Hc) * a.n_tiles >= kSmallWorkgroupsFrom * fp::compute_units()) {
+      constexpr int BM4 = (4 / G) * 32;
+      a.n_tiles = (a.Lq + BM4 - 1) / BM4;
+      dim3 grid4(a.Hc, a.n_tiles, 1);
+      if (a.pd.shift >= 0)
+        hipLaunchKernelGGL((paged_prefill_kernel<E, D, G, true, 4>), grid4, dim3(256), 0, st, a);
+      else
+        hipLaunchKernelGGL((paged_prefill_kernel<E, D, G, false, 4>), grid4, dim3(256), 0, st, a);
+      return;
+    }
   }
   dim3 grid(a.Hc, a.n_tiles, shares);
   if (a.pd.shift >= 0)

@@ -265,3 +265,40 @@ def test_every_kernel_instance(dtype, D, G, P):
     q, k, v, out, lse = prefill_through_api(st, ids, bidx, pos, G, dtype, 1)
     eo, el = O.prefill_attention_packed(f64(q), f64(k), f64(v), bidx[None], ids[None], SOI, EOI)
     assert_close(out, lse, eo, el, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)
+@pytest.mark.parametrize("G,Hc", [(1, 16), (2, 8), (4, 4)])
+@pytest.mark.parametrize("P", [128, 24], ids=["page-holds-tile", "odd-page"])
+def test_head_dim_64_launch_of_a_workgroup_per_cu_and_more(dtype, G, Hc, P):
+    """At head_dim 64 a launch that fills the GPU goes out as workgroups of four wavefronts (two to a CU):
+    4096 rows x 16 query heads, 8 sequences packed without padding, image spans, prefixes already in pages.
+    Sampled rows against the oracle; a padding stretch in the middle of the row."""
+    gen = torch.Generator().manual_seed(64 + G)
+    n_seq, chunk = 8, 500
+    prefixes = [int(x) for x in torch.randint(0, 700, (n_seq,), generator=gen)]
+    st = PagedState(64 + G, n_pages=sum(-(-(p + chunk) // P) for p in prefixes) + 8, page_size=P, max_batch=n_seq + 2,
+                    Hc=Hc, D=64, dtype=dtype)
+    st.cache.kv_cache.view(-1).normal_(generator=torch.Generator(device=DEV).manual_seed(1))
+    bidx, lim = [], []
+    for i, p in enumerate(prefixes):
+        b = st.add_sequence(p + chunk)
+        span = 200 if i % 2 else 0  # rows of the chunk's first `span` positions see the whole span
+        bidx += [b] * chunk
+        lim += [max(p + t + 1, p + span) for t in range(chunk)]
+        if i == 3:
+            bidx += [0] * 96
+            lim += [0] * 96
+    Lq = len(bidx)
+    assert Lq == 4096
+    q = randn(st.gen, (1, Hc * G, Lq, 64), dtype).to(DEV)
+    pk, pv = st.pool_planes()
+    bidx_t = torch.tensor(bidx, dtype=torch.int64, device=DEV)
+    lim_t = torch.tensor(lim, dtype=torch.int32, device=DEV)
+    out, lse = ops.paged_prefill(q, pk, pv, st.cache.page_table, bidx_t, lim_t, P)
+    rows = np.arange(0, Lq, 29)
+    eo, el = O.prefill_attention_paged(f64(q[:, :, rows]), f64(pk), f64(pv), st.mirror.page_table, np.array(bidx)[rows],
+                                       None, np.array(lim)[rows], P)
+    assert_close(out[:, :, rows], lse[:, :, rows], eo, el, dtype)
+    pad = np.flatnonzero(np.array(bidx) == 0)
+    assert not f64(out)[:, :, pad].any() and np.isneginf(f64(lse)[:, :, pad]).all()
