@@ -149,7 +149,7 @@ struct Swizzle {
 // travel from L2 into LDS (64 B per cycle and CU, and a wavefront waits at its load instructions
 // while that path is busy) are shared by all of them.
 template <typename E, int D, int G, bool kPow2, int W = kWaves>
-__global__ __launch_bounds__(W * 64, 2) void paged_prefill_kernel(const PrefillArgs a) {
+__global__ __launch_bounds__(W * 64, (W == 4 && D == 64 ? 3 : 2)) void paged_prefill_kernel(const PrefillArgs a) {
   constexpr int kThreads = W * 64;  // shadows the file-scope constant: W wavefronts per workgroup
   using SW = Swizzle<D>;
   constexpr int MB = 1;                    // 32-row blocks per wavefront
@@ -750,8 +750,10 @@ void launch_group(const PrefillArgs& a0, void* workspace, int64_t workspace_byte
   // wavefronts, two to a CU.  A staged K/V tile then serves half as many query rows, but at 128-byte rows the
   // staging is cheap, the softmax (which does not shrink with head_dim) is what a step waits for, and two
   // independent workgroups per CU fill each other's barrier and set-up gaps: 8 x 512-row chunks 85 us against
-  // 91 us, the same 8 sequences whole 350 us against 370 us.  At head_dim 128 the same split is slower
-  // (whole sequences 564 us against 485 us): the staging path is the limit there.
+  // 91 us, the same 8 sequences whole 350 us against 370 us - and 316 us with three such workgroups per CU
+  // (the kernel is compiled for 168 registers there, a handful of values spilled outside the tile loop).
+  // At head_dim 128 the same split is slower (whole sequences 564 us against 485 us): the staging path is
+  // the limit there, and its 242 registers allow two wavefronts per SIMD at most.
   if constexpr (G <= 4 && D == 64) {
     if (shares == 1 && static_cast<int64_t>(a.Hc) * a.n_tiles >= kSmallWorkgroupsFrom * fp::compute_units()) {
       constexpr int BM4 = (4 / G) * 32;
