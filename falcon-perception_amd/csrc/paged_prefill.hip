@@ -10,7 +10,7 @@
 //
 // MFMA-bound.  A workgroup of 8 wavefronts owns one cache head and 256 / G consecutive packed
 // query rows of each of its G query heads; a wavefront owns 32 rows of one query head.  (Large launches
-// at head_dim 64 use workgroups of 4 wavefronts and 128 / G rows, two to a CU.)
+// at head_dim 64 use workgroups of 4 wavefronts and 128 / G rows, three to a CU.)
 //   S^T = K Q^T  (v_mfma_f32_32x32x16): keys are the M rows, queries the N columns, so a
 //         lane holds scores of ONE query and softmax row reductions stay in registers
 //         (plus one exchange between the two lane halves).
@@ -747,7 +747,7 @@ void launch_group(const PrefillArgs& a0, void* workspace, int64_t workspace_byte
     a.ws_acc = reinterpret_cast<short*>(a.ws_ml + static_cast<int64_t>(shares) * a.Lq * a.Hq * 2);
   }
   // head_dim 64: a launch with at least one eight-wavefront workgroup per CU goes out as workgroups of four
-  // wavefronts, two to a CU.  A staged K/V tile then serves half as many query rows, but at 128-byte rows the
+  // wavefronts, up to three to a CU.  A staged K/V tile then serves half as many query rows, but at 128-byte rows the
   // staging is cheap, the softmax (which does not shrink with head_dim) is what a step waits for, and two
   // independent workgroups per CU fill each other's barrier and set-up gaps: 8 x 512-row chunks 85 us against
   // 91 us, the same 8 sequences whole 350 us against 370 us - and 316 us with three such workgroups per CU
