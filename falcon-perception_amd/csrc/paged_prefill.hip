@@ -715,7 +715,6 @@ __global__ __launch_bounds__(kMergeRows * 64) void paged_prefill_merge_kernel(co
 }
 
 constexpr int kMaxKeyShares = 8;
-constexpr int kSmallWorkgroupsFrom = 1;  // eight-wavefront workgroups per CU from which a head_dim 64 launch uses four-wavefront ones
 
 // Key shares for a launch of `wgs` workgroups.  bf16 / f16: a launch that would leave at least half of the
 // CUs idle is cut along the keys until every CU has a workgroup.  (With about one workgroup per CU
@@ -746,16 +745,17 @@ void launch_group(const PrefillArgs& a0, void* workspace, int64_t workspace_byte
     a.ws_ml = static_cast<float*>(workspace);
     a.ws_acc = reinterpret_cast<short*>(a.ws_ml + static_cast<int64_t>(shares) * a.Lq * a.Hq * 2);
   }
-  // head_dim 64: a launch with at least one eight-wavefront workgroup per CU goes out as workgroups of four
-  // wavefronts, up to three to a CU.  A staged K/V tile then serves half as many query rows, but at 128-byte rows the
-  // staging is cheap, the softmax (which does not shrink with head_dim) is what a step waits for, and two
-  // independent workgroups per CU fill each other's barrier and set-up gaps: 8 x 512-row chunks 85 us against
-  // 91 us, the same 8 sequences whole 350 us against 370 us - and 316 us with three such workgroups per CU
-  // (the kernel is compiled for 168 registers there, a handful of values spilled outside the tile loop).
+  // head_dim 64: a launch that is not cut along the keys goes out as workgroups of four wavefronts, up to
+  // three to a CU.  A staged K/V tile then serves half as many query rows, but at 128-byte rows the staging is
+  // cheap, the softmax (which does not shrink with head_dim) is what a step waits for, and independent
+  // workgroups on a CU fill each other's barrier and set-up gaps: 8 x 512-row chunks 85 us against 91 us, the
+  // same 8 sequences whole 350 us against 370 us with two per CU and 316 us with three (the instance is
+  // compiled for 168 registers, a handful of values spilled outside the tile loop); 6 chunks 85 us against
+  // 91 us, and where no workspace allows the cut along the keys, 1 / 4 chunks 59 / 72 us against 74 / 90 us.
   // At head_dim 128 the same split is slower (whole sequences 564 us against 485 us): the staging path is
   // the limit there, and its 242 registers allow two wavefronts per SIMD at most.
   if constexpr (G <= 4 && D == 64) {
-    if (shares == 1 && static_cast<int64_t>(a.Hc) * a.n_tiles >= kSmallWorkgroupsFrom * fp::compute_units()) {
+    if (shares == 1) {
       constexpr int BM4 = (4 / G) * 32;
       a.n_tiles = (a.Lq + BM4 - 1) / BM4;
       dim3 grid4(a.Hc, a.n_tiles, 1);
