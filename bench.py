@@ -586,8 +586,14 @@ def prefill_rate(steps: int = 10, name: str = "cfg3") -> dict:
             "cfg3d64": "cfg3 at head_dim 64 (the reference's OCR and 300M variants)",
             "cfg3one": "one sequence alone: paged prefix 4096, 512-token chunk, 16 q / 8 kv heads, D 128 "
                        "(cut along the keys into 8 shares + merge pass)"}[name]
+    # key tiles (64 keys) each 128-row query tile walks: a launch of about one workgroup per CU lasts as long as
+    # its longest workgroup, so longest / mean bounds what such a launch can reach of a balanced one's rate
+    lim = case.row_limit.view(-1, 128).max(dim=1).values.float()
+    tiles = torch.ceil(lim[lim > 0] / 64)
     res = {"workload": what, "query_rows": int(case.q.shape[2]), "paged_prefill_ms": ms, "tflops": tf,
-           "chunk_append_ms": ms_a, "flops": case.flops()}
+           "chunk_append_ms": ms_a, "flops": case.flops(),
+           "key_tiles_per_query_tile": {"longest": int(tiles.max()), "mean": round(float(tiles.mean()), 1),
+                                        "query_tiles_per_head": int(tiles.numel())}}
     if case.q.dtype == torch.float32:
         res["frac_of_f32_mfma_peak"] = tf / MFMA_F32_PEAK_TFLOPS
     else:
