@@ -32,6 +32,8 @@
 #include <hip/hip_fp16.h>
 #include <math.h>
 
+#include <type_traits>
+
 namespace {
 
 constexpr int kWaves = 8;
@@ -148,7 +150,7 @@ struct Swizzle {
 // 32 query rows: every head of the group works from the same staged K/V tile, so the bytes that
 // travel from L2 into LDS (64 B per cycle and CU, and a wavefront waits at its load instructions
 // while that path is busy) are shared by all of them.
-template <typename E, int D, int G, bool kPow2, int W = kWaves>
+template <typename E, int D, int G, bool kPow2, int W = kWaves, bool kBounded = false>
 __global__ __launch_bounds__(W * 64, (W == 4 && D == 64 ? 3 : 2)) void paged_prefill_kernel(const PrefillArgs a) {
   constexpr int kThreads = W * 64;  // shadows the file-scope constant: W wavefronts per workgroup
   using SW = Swizzle<D>;
@@ -209,6 +211,13 @@ __global__ __launch_bounds__(W * 64, (W == 4 && D == 64 ? 3 : 2)) void paged_pre
     for (int ds = 0; ds < DS; ++ds) {
       v4u w = {0, 0, 0, 0};
       if (in) w = *reinterpret_cast<const v4u*>(a.q + row[mb] * a.qs_row + hq * a.qs_h + (16 * ds + 8 * half) * 2);
+      if constexpr (kBounded) {
+        // bounded scores: Q carries scale * log2(e), so that the matrix product leaves the exponent itself
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          w[c] = E::pack2(E::to_float(static_cast<short>(w[c] & 0xffffu)) * a.qscale,
+                          E::to_float(static_cast<short>(w[c] >> 16)) * a.qscale);
+      }
       qreg[mb][ds] = __builtin_bit_cast(s16x8, w);
     }
   }
@@ -317,7 +326,7 @@ __global__ __launch_bounds__(W * 64, (W == 4 && D == 64 ? 3 : 2)) void paged_pre
     float m_run[MB], l_run[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
-      m_run[mb] = -INFINITY;
+      m_run[mb] = kBounded ? 0.f : -INFINITY;  // bounded scores: the reference point of the exponentials is 0 throughout
       l_run[mb] = 0.f;
 #pragma unroll
       for (int db = 0; db < DB; ++db) o_acc[mb][db] = kZero16;
@@ -552,6 +561,25 @@ __global__ __launch_bounds__(W * 64, (W == 4 && D == 64 ? 3 : 2)) void paged_pre
               sc[x] = key < rel ? sc[x] : -INFINITY;
             }
           }
+          if constexpr (kBounded) {
+            // |score| is bounded by the caller's declaration: exp2 of the score itself neither overflows nor
+            // vanishes in fp32 / bf16, so there is no running maximum, no exchange between the lane halves,
+            // no vote and no rescale: exponential, pack, row sum
+            float part[4] = {0.f, 0.f, 0.f, 0.f};
+            uint32_t pw[16];
+#pragma unroll
+            for (int x = 0; x < 32; x += 2) {
+              const float p0 = fast_exp2(sc[x]);
+              const float p1 = fast_exp2(sc[x + 1]);
+              pw[x >> 1] = E::pack2(p0, p1);
+              part[(x >> 1) & 3] += p0 + p1;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              p_op[mb][j] = __builtin_bit_cast(s16x8, v4u{pw[4 * j], pw[4 * j + 1], pw[4 * j + 2], pw[4 * j + 3]});
+            l_run[mb] += (part[0] + part[1]) + (part[2] + part[3]);
+            continue;
+          }
           // four independent chains: one wavefront alone issues a dependent instruction every ~8 cycles
           float mx4[4] = {sc[0], sc[1], sc[2], sc[3]};
 #pragma unroll
@@ -734,9 +762,39 @@ int64_t share_bytes(int shares, int Lq, int Hq, int D, int elem) {
   return shares <= 1 ? 0 : static_cast<int64_t>(shares) * Lq * Hq * (static_cast<int64_t>(D) * elem + 8);
 }
 
+// Scores the caller bounds (|scale * q.k| <= score_bound, natural units) take the kernel instance without a
+// running maximum.  bf16 only: the probabilities span 2^(+-bound * log2 e), which bf16 (fp32's exponent
+// range) holds and f16 does not; the limit keeps row sums over 2^31 keys and the accumulators inside fp32.
+constexpr float kMaxScoreBound = 40.f;
+
+template <typename E>
+bool bounded_path(float score_bound) {
+  return std::is_same<E, BF16>::value && score_bound > 0.f && score_bound <= kMaxScoreBound;
+}
+
+template <typename E, int D, int G, bool kPow2, int W, bool kBounded>
+void launch_instance(const PrefillArgs& a, dim3 grid, hipStream_t st) {
+  hipLaunchKernelGGL((paged_prefill_kernel<E, D, G, kPow2, W, kBounded>), grid, dim3(W * 64), 0, st, a);
+}
+
+template <typename E, int D, int G, int W>
+void launch_main(const PrefillArgs& a, dim3 grid, bool bounded, hipStream_t st) {
+  const bool pow2 = a.pd.shift >= 0;
+  if constexpr (std::is_same<E, BF16>::value) {
+    if (bounded) {
+      if (pow2) launch_instance<E, D, G, true, W, true>(a, grid, st);
+      else launch_instance<E, D, G, false, W, true>(a, grid, st);
+      return;
+    }
+  }
+  if (pow2) launch_instance<E, D, G, true, W, false>(a, grid, st);
+  else launch_instance<E, D, G, false, W, false>(a, grid, st);
+}
+
 template <typename E, int D, int G>
-void launch_group(const PrefillArgs& a0, void* workspace, int64_t workspace_bytes, hipStream_t st) {
+void launch_group(const PrefillArgs& a0, float score_bound, void* workspace, int64_t workspace_bytes, hipStream_t st) {
   PrefillArgs a = a0;
+  const bool bounded = bounded_path<E>(score_bound);
   constexpr int BM = (kWaves / G) * 32;
   a.n_tiles = (a.Lq + BM - 1) / BM;
   int shares = workspace ? key_shares_for(static_cast<int64_t>(a.Hc) * a.n_tiles, FP_DTYPE_BF16) : 1;  // f16 alike
@@ -758,19 +816,11 @@ void launch_group(const PrefillArgs& a0, void* workspace, int64_t workspace_byte
     if (shares == 1) {
       constexpr int BM4 = (4 / G) * 32;
       a.n_tiles = (a.Lq + BM4 - 1) / BM4;
-      dim3 grid4(a.Hc, a.n_tiles, 1);
-      if (a.pd.shift >= 0)
-        hipLaunchKernelGGL((paged_prefill_kernel<E, D, G, true, 4>), grid4, dim3(256), 0, st, a);
-      else
-        hipLaunchKernelGGL((paged_prefill_kernel<E, D, G, false, 4>), grid4, dim3(256), 0, st, a);
+      launch_main<E, D, G, 4>(a, dim3(a.Hc, a.n_tiles, 1), bounded, st);
       return;
     }
   }
-  dim3 grid(a.Hc, a.n_tiles, shares);
-  if (a.pd.shift >= 0)
-    hipLaunchKernelGGL((paged_prefill_kernel<E, D, G, true>), grid, dim3(kThreads), 0, st, a);
-  else
-    hipLaunchKernelGGL((paged_prefill_kernel<E, D, G, false>), grid, dim3(kThreads), 0, st, a);
+  launch_main<E, D, G, kWaves>(a, dim3(a.Hc, a.n_tiles, shares), bounded, st);
   if (shares > 1) {
     const int64_t items = static_cast<int64_t>(a.Lq) * a.Hq;
     hipLaunchKernelGGL((paged_prefill_merge_kernel<E, D>), dim3(static_cast<unsigned>((items + kMergeRows - 1) / kMergeRows)),
@@ -779,12 +829,12 @@ void launch_group(const PrefillArgs& a0, void* workspace, int64_t workspace_byte
 }
 
 template <typename E, int D>
-int launch(const PrefillArgs& a, void* ws, int64_t ws_bytes, hipStream_t st) {
+int launch(const PrefillArgs& a, float score_bound, void* ws, int64_t ws_bytes, hipStream_t st) {
   switch (a.Hq / a.Hc) {
-    case 1: launch_group<E, D, 1>(a, ws, ws_bytes, st); return FP_OK;
-    case 2: launch_group<E, D, 2>(a, ws, ws_bytes, st); return FP_OK;
-    case 4: launch_group<E, D, 4>(a, ws, ws_bytes, st); return FP_OK;
-    case 8: launch_group<E, D, 8>(a, ws, ws_bytes, st); return FP_OK;
+    case 1: launch_group<E, D, 1>(a, score_bound, ws, ws_bytes, st); return FP_OK;
+    case 2: launch_group<E, D, 2>(a, score_bound, ws, ws_bytes, st); return FP_OK;
+    case 4: launch_group<E, D, 4>(a, score_bound, ws, ws_bytes, st); return FP_OK;
+    case 8: launch_group<E, D, 8>(a, score_bound, ws, ws_bytes, st); return FP_OK;
     default: return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill: Hq/Hc = %d (supported: 1, 2, 4, 8)", a.Hq / a.Hc);
   }
 }
@@ -797,8 +847,8 @@ extern "C" int fp_paged_prefill(const void* q, int64_t q_stride_row, int64_t q_s
                                 int64_t out_stride_row, int64_t out_stride_h, float* lse, const float* sinks,
                                 int32_t Lq, int32_t Hq,
                                 int32_t Hc, int32_t D, int32_t page_size, int32_t n_pages, int32_t max_batch,
-                                int64_t n_slots, float scale, int dtype, void* workspace, int64_t workspace_bytes,
-                                void* stream) {
+                                int64_t n_slots, float scale, float score_bound, int dtype, void* workspace,
+                                int64_t workspace_bytes, void* stream) {
   if (dtype != FP_DTYPE_BF16 && dtype != FP_DTYPE_F16 && dtype != FP_DTYPE_F32)
     return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill: unknown dtype %d", dtype);
   if (D != 64 && D != 128) return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill: head_dim %d (supported: 64, 128)", D);
@@ -838,9 +888,11 @@ extern "C" int fp_paged_prefill(const void* q, int64_t q_stride_row, int64_t q_s
   hipStream_t st = static_cast<hipStream_t>(stream);
   int rc;
   if (dtype == FP_DTYPE_BF16)
-    rc = D == 64 ? launch<BF16, 64>(a, workspace, workspace_bytes, st) : launch<BF16, 128>(a, workspace, workspace_bytes, st);
+    rc = D == 64 ? launch<BF16, 64>(a, score_bound, workspace, workspace_bytes, st)
+                 : launch<BF16, 128>(a, score_bound, workspace, workspace_bytes, st);
   else
-    rc = D == 64 ? launch<F16, 64>(a, workspace, workspace_bytes, st) : launch<F16, 128>(a, workspace, workspace_bytes, st);
+    rc = D == 64 ? launch<F16, 64>(a, score_bound, workspace, workspace_bytes, st)
+                 : launch<F16, 128>(a, score_bound, workspace, workspace_bytes, st);
   if (rc != FP_OK) return rc;
   return fp::check_launch("fp_paged_prefill");
 }

@@ -13,7 +13,7 @@ from .paged_attention import PagedKVCache  # noqa: F401
 __all__ = ["KVCacheBase", "PagedKVCache", "attention", "kv_cache", "ops", "paged_attention", "install"]
 
 
-def install(kv_rep: int = 1) -> None:
+def install(kv_rep: int = 1, qk_norm: bool = False) -> None:
     """Serve the reference's module names from this package.
 
     After `install()`, `import falcon_perception.paged_attention`,
@@ -28,12 +28,18 @@ def install(kv_rep: int = 1) -> None:
     reference's `repeat_kv` hands to `insert_kv` (`model.py:112-116`): decode then reads V once
     per group.  The engine builds its cache with `n_heads` heads (`paged_inference.py:321-330`)
     and never says so itself; left at 1, every cached head is read in full.
+
+    `qk_norm=True` states that the model RMS-normalises q and k without a weight before the rotary
+    embedding, as every variant of the reference does (`model.py:110-116`): |q| = |k| = sqrt(head_dim),
+    so the attention scores are bounded and the bf16 prefill kernel runs its softmax without a running
+    maximum (`score_bound` of `fp_paged_prefill`).  Leave it off for a model with learned norm weights.
     """
     import sys
 
     if kv_rep < 1:
         raise ValueError("kv_rep must be at least 1")
     PagedKVCache.default_kv_rep = int(kv_rep)
+    PagedKVCache.default_qk_normalised = bool(qk_norm)
     sys.modules["falcon_perception.kv_cache"] = kv_cache
     sys.modules["falcon_perception.paged_attention"] = paged_attention
     sys.modules["falcon_perception.attention"] = attention

@@ -280,6 +280,7 @@ def compiled_flex_attn_prefill(q: Tensor, k: Tensor, v: Tensor, score_mod=None, 
         q, pool_k, pool_v, cache.page_table, step.batch_idx,
         block_mask.row_limit(step.input_pos, step.layer_id), cache.page_size, scale=scale, sinks=sinks,
         workspace=cache.prefill_workspace(q.shape[2], q.shape[1], q.shape[3], pool_k.shape[0], q.dtype),
+        score_bound=cache.score_bound(q.shape[3], scale),
     )
     return _result(out, lse, return_aux, return_lse)
 

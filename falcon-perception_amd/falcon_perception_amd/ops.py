@@ -325,12 +325,15 @@ def hybrid_row_limits(input_ids: Tensor, soi_id: int, eoi_id: int, batch_idx: Te
 def paged_prefill(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor, batch_idx: Tensor,
                   row_limit: Tensor, page_size: int, *, scale: float | None = None,
                   out: Tensor | None = None, lse: Tensor | None = None,
-                  sinks: Tensor | None = None, workspace: Tensor | None | bool = None) -> tuple[Tensor, Tensor]:
+                  sinks: Tensor | None = None, workspace: Tensor | None | bool = None,
+                  score_bound: float = 0.0) -> tuple[Tensor, Tensor]:
     """Chunked-prefill attention over the paged cache.  q [1, Hq, Lq, D]; row r sees keys
     0..row_limit[r]-1 of sequence batch_idx[r]; returns out like q, lse [1, Hq, Lq].
     `sinks` [Hq] float32 gates the output as in `paged_decode`.  `workspace`: a uint8 tensor of
     `prefill_workspace_bytes(...)` bytes lets a launch too small for the GPU be cut along the keys as
-    well; None allocates one when the shape calls for it, False runs without."""
+    well; None allocates one when the shape calls for it, False runs without.  `score_bound` > 0 is the
+    caller's guarantee that |scale * q.k| never exceeds it (sqrt(D) for the model's normalised q and k): the
+    bf16 kernel then runs its softmax without a running maximum."""
     N.require_cuda(q, pool_k, pool_v, page_table, batch_idx, row_limit, out, lse)
     one, Hq, Lq, D = q.shape
     if one != 1:
@@ -369,7 +372,7 @@ def paged_prefill(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor,
         page_table.data_ptr(), page_table.stride(0), batch_idx.data_ptr(),
         row_limit.data_ptr(), out.data_ptr(), out.stride(2), out.stride(1), lse.data_ptr(),
         _sinks_ptr(sinks, Hq, q.device), Lq, Hq, Hc, D, page_size, page_table.shape[1], page_table.shape[0], n_slots,
-        scale, N.dtype_code(q.dtype), ws_ptr, ws_bytes, N.stream_ptr(q.device))
+        scale, float(score_bound), N.dtype_code(q.dtype), ws_ptr, ws_bytes, N.stream_ptr(q.device))
     N.check(rc, "fp_paged_prefill")
     return out, lse
 

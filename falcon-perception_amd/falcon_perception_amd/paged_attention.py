@@ -53,6 +53,7 @@ class PagedKVCache(KVCacheBase):
     """
 
     default_kv_rep = 1  # kv_rep of caches created from now on, see `falcon_perception_amd.install`
+    default_qk_normalised = False  # likewise: whether the q and k rows the model produces have norm sqrt(head_dim)
 
     def __init__(self, n_pages: int, page_size: int, max_batch_size: int, n_heads: int, head_dim: int,
                  num_layers: int, dtype: torch.dtype, device: str | torch.device = "cuda",
@@ -88,6 +89,11 @@ class PagedKVCache(KVCacheBase):
         # default (`falcon_perception_amd.install(kv_rep=...)` sets it for an engine that is not edited) when
         # it divides this cache's head count.
         self.kv_rep = self.default_kv_rep if n_heads % self.default_kv_rep == 0 else 1
+        # Whether every q and k row has norm sqrt(head_dim): the reference's model RMS-normalises both without a
+        # weight and rotates them (model.py:110-116).  |scale * q.k| is then at most scale * head_dim, and the
+        # bf16 prefill kernel runs its softmax without a running maximum (`score_bound`).  Set by
+        # `insert_qkv_norm_rope`, which does the normalisation itself, or by `install(qk_norm=True)`.
+        self.qk_normalised = self.default_qk_normalised
 
         # what the attention callables need from the step in flight
         self.last_decode_step: StepMeta | None = None
@@ -163,6 +169,7 @@ class PagedKVCache(KVCacheBase):
             assert B == 1 and batch_idx.shape == (1, S), "a prefill step is one packed row"
         q = ops.qkv_norm_rope_append(xq, xk, xv, freqs_cis, freqs_cis_2d, *self._planes[layer_id], self.page_table,
                                      batch_idx, input_pos, self.page_size, clamp_negative=decode)
+        self.qk_normalised = True  # every row this call wrote or returned has norm sqrt(head_dim)
         if decode:
             self.last_decode_step = StepMeta(layer_id, input_pos, batch_idx)
         else:
@@ -352,6 +359,13 @@ class PagedKVCache(KVCacheBase):
             hit = (need, self.decode_split_tokens(B, Hc, max_context))
             self._decode_launch[key] = hit
         return (self._workspace if hit[0] else None), hit[1]
+
+    def score_bound(self, head_dim: int, scale: float | None) -> float:
+        """Bound of |scale * q.k| the prefill kernel may rely on: 0 (unknown) unless q and k are normalised;
+        then scale * head_dim with a tenth of slack for the roundings after the norm and the rotation."""
+        if not self.qk_normalised:
+            return 0.0
+        return 1.1 * head_dim * (head_dim ** -0.5 if scale is None else abs(scale))
 
     def prefill_workspace(self, Lq: int, Hq: int, D: int, Hc: int, dtype: torch.dtype):
         """Scratch with which the prefill kernel cuts a small launch along the keys as well, owned by the

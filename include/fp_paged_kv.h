@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define FP_ABI_VERSION 4
+#define FP_ABI_VERSION 5
 
 /* element types of pool / q / k / v */
 #define FP_DTYPE_F32 0
@@ -358,6 +358,16 @@ int fp_hybrid_row_limits(const int64_t* input_ids, const int64_t* batch_idx,
  *              every such key must already be in the pages
  *   out        [Lq, Hq, D] view, strides (row, head); lse [Hq, Lq] float32
  *   sinks      NULL, or [Hq] float32 attention-sink logits, as in fp_paged_decode
+ *   score_bound  0 when nothing is known about the scores; otherwise the caller's guarantee that
+ *              |scale * q.k| <= score_bound for every visible (query, key) pair of the launch.  The
+ *              reference's model RMS-normalises q and k without a weight and rotates them
+ *              (model.py:110-116), so |q| = |k| = sqrt(D) and score_bound = sqrt(D) holds by
+ *              construction.  With 0 < score_bound <= 40 the bf16 kernel drops the running maximum of
+ *              the online softmax: Q is multiplied by scale * log2(e) when it is loaded (and rounded to
+ *              bf16 again), and the probabilities are exp2 of the matrix product itself, referred to the
+ *              fixed point 0.  Results agree with the unbounded path within bf16 rounding.  A bound
+ *              the data breaks gives wrong results only once exp2(score * log2 e) leaves fp32's
+ *              range.  f16 and fp32 ignore the argument.
  *   workspace  NULL, or workspace_bytes bytes of device memory, 16-byte aligned (no need to clear it).
  *              A launch with fewer workgroups than the GPU needs (few query rows, few heads) is then
  *              also cut along the keys: up to 8 workgroups share a query tile, each takes an equal part
@@ -377,7 +387,7 @@ int fp_paged_prefill(const void* q, int64_t q_stride_row, int64_t q_stride_h,
                      float* lse, const float* sinks,
                      int32_t Lq, int32_t Hq, int32_t Hc, int32_t D,
                      int32_t page_size, int32_t n_pages, int32_t max_batch,
-                     int64_t n_slots, float scale, int dtype,
+                     int64_t n_slots, float scale, float score_bound, int dtype,
                      void* workspace, int64_t workspace_bytes,
                      void* stream);
 

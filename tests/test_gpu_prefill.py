@@ -17,13 +17,18 @@ pytestmark = pytest.mark.gpu
 TOL = {torch.bfloat16: (2e-2, 1e-2), torch.float16: (4e-3, 4e-3), torch.float32: (2e-5, 2e-5)}
 
 
-def assert_close(out, lse, eo, el, dtype, rows=None):
+# The bounded-score path multiplies Q by scale * log2(e) and rounds it to bf16 once more: a score, and with it
+# the lse of a row that sees few keys, moves by up to |q||k| 2^-9 / sqrt(3 D) ~ 1e-3 per standard deviation.
+BOUNDED_LSE_ATOL = 5e-3
+
+
+def assert_close(out, lse, eo, el, dtype, rows=None, lse_atol=None):
     atol, rtol = TOL[dtype]
     go, gl = f64(out), f64(lse)
     if rows is not None:
         go, gl, eo, el = go[:, :, rows], gl[:, :, rows], eo[:, :, rows], el[:, :, rows]
     np.testing.assert_allclose(go, eo, atol=atol, rtol=rtol)
-    np.testing.assert_allclose(gl, el, atol=max(atol * 0.1, 1e-4), rtol=rtol)
+    np.testing.assert_allclose(gl, el, atol=lse_atol or max(atol * 0.1, 1e-4), rtol=rtol)
 
 
 def prefill_through_api(st, ids, bidx, pos, Hq, dtype, pad_to):
@@ -153,6 +158,7 @@ def test_cfg3_chunked_prefill_shape():
     import bench
 
     case = bench.make_prefill_case("cfg3", device=DEV)
+    case.use_bound = False  # the online softmax with its running maximum
     out, lse = case.run()
     pk, pv = case.pool_k.float().cpu().numpy(), case.pool_v.float().cpu().numpy()
     bidx = case.batch_idx.cpu().numpy().reshape(-1)
@@ -302,3 +308,109 @@ def test_head_dim_64_launch_of_a_workgroup_per_cu_and_more(dtype, G, Hc, P):
     assert_close(out[:, :, rows], lse[:, :, rows], eo, el, dtype)
     pad = np.flatnonzero(np.array(bidx) == 0)
     assert not f64(out)[:, :, pad].any() and np.isneginf(f64(lse)[:, :, pad]).all()
+
+
+# ---- bounded scores: the bf16 softmax without a running maximum -------------------------------------
+
+def rms_normalised(gen, shape, dtype):
+    """Rows of norm sqrt(D), as the model's weightless RMS norm leaves q and k (model.py:110-116), rounded to dtype."""
+    x = torch.randn(shape, generator=gen, dtype=torch.float32)
+    return (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True))).to(dtype)
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("G", [1, 2, 4, 8])
+@pytest.mark.parametrize("P", [64, 16, 24], ids=["page-holds-tile", "small-page", "odd-page"])
+def test_bounded_scores_every_kernel_instance(D, G, P):
+    """The instances of the bf16 kernel that take the caller's score bound, one packed step each, through the
+    drop-in callables: a cache that knows its q and k rows are normalised declares 1.1 * sqrt(D)."""
+    dtype = torch.bfloat16
+    layout = layout_for([(1, 70, 0, 0), (2, 9, 60, 45)])
+    ids, bidx, pos = repack(layout, 1)
+    st = PagedState(140 + G, n_pages=24, page_size=P, max_batch=4, Hc=1, D=D, dtype=dtype)
+    for slot in (1, 2):
+        st.add_sequence(int((bidx == slot).sum()))
+    cache, L = st.cache, len(ids)
+    cache.qk_normalised = True
+    assert cache.score_bound(D, None) == pytest.approx(1.1 * D ** 0.5)
+    dev = lambda a: torch.from_numpy(a)[None].to(DEV)
+    mask = cache.create_prefill_blockmask(dev(bidx), dev(ids), SOI, EOI)
+    k = rms_normalised(st.gen, (1, 1, L, D), dtype)
+    v = randn(st.gen, (1, 1, L, D), dtype)
+    q = rms_normalised(st.gen, (1, G, L, D), dtype)
+    K, V = cache.insert_kv(0, k.to(DEV), v.to(DEV), input_pos=dev(pos), batch_idx=dev(bidx))
+    out, aux = A.compiled_flex_attn_prefill(q.to(DEV), K, V, block_mask=mask, return_aux=AuxRequest(lse=True))
+    eo, el = O.prefill_attention_packed(f64(q), f64(k), f64(v), bidx[None], ids[None], SOI, EOI)
+    assert_close(out, aux.lse, eo, el, dtype, lse_atol=BOUNDED_LSE_ATOL)
+
+
+@pytest.mark.parametrize("bound,peak", [(12.0, 11.0), (40.0, 38.0), (41.0, 38.0), (0.0, 38.0)])
+def test_bounded_scores_over_a_wide_range(bound, peak):
+    """Scores spread over +-peak (natural units): with the fixed reference point the probabilities span
+    2^(+-peak * log2 e) and must survive in bf16 / fp32 without a running maximum; rows whose largest score is
+    far below zero keep their precision.  A bound above the kernel's limit of 40, or none, takes the ordinary path."""
+    dtype, D, P, L = torch.bfloat16, 128, 64, 300
+    st = PagedState(150, n_pages=12, page_size=P, max_batch=3, Hc=1, D=D, dtype=dtype)
+    b = st.add_sequence(L)
+    gen = st.gen
+    # keys along one direction with lengths that put scale * q.k anywhere in [-peak, peak]
+    u = torch.randn(D, generator=gen)
+    u /= u.norm()
+    k = (u[None] * (torch.rand(L, 1, generator=gen) * 2 - 1) * 16 + 0.05 * torch.randn(L, D, generator=gen)).to(dtype)
+    q = (u[None] * (torch.rand(L, 1, generator=gen) * 2 - 1) * (peak * D ** 0.5 / 16.2)
+         + 0.05 * torch.randn(L, D, generator=gen)).to(dtype)
+    assert (q.float() @ k.float().T).abs().max() / D ** 0.5 <= peak
+    v = randn(gen, (L, D), dtype)
+    bt, pt = torch.full((1, L), b, dtype=torch.int64), torch.arange(L)[None]
+    st.cache.insert_kv(0, k.view(1, 1, L, D).to(DEV), v.view(1, 1, L, D).to(DEV), input_pos=pt.to(DEV), batch_idx=bt.to(DEV))
+    lim = torch.arange(1, L + 1, dtype=torch.int32)
+    pk, pv = st.pool_planes()
+    q4 = q.view(1, 1, L, D)
+    out, lse = ops.paged_prefill(q4.to(DEV), pk, pv, st.cache.page_table, bt.view(-1).to(DEV), lim.to(DEV), P,
+                                 score_bound=bound)
+    eo, el = O.prefill_attention_paged(f64(q4), f64(pk), f64(pv), st.mirror.page_table, bt.view(-1).numpy(), None,
+                                       lim.numpy(), P)
+    assert_close(out, lse, eo, el, dtype, lse_atol=BOUNDED_LSE_ATOL)
+
+
+def test_bounded_scores_key_shares_and_f16():
+    """A launch small enough to be cut along the keys (one 300-row chunk over a 3000-token prefix) with the bound
+    declared: the shares' partial results all refer to the fixed point 0 and the merge pass combines them as
+    before.  f16 ignores the bound."""
+    D, P, prefix, chunk = 128, 128, 3000, 300
+    for dtype in (torch.bfloat16, torch.float16):
+        st = PagedState(151, n_pages=32, page_size=P, max_batch=3, Hc=2, D=D, dtype=dtype)
+        b = st.add_sequence(prefix + chunk)
+        L = prefix + chunk
+        k = rms_normalised(st.gen, (1, 2, L, D), dtype)
+        v = randn(st.gen, (1, 2, L, D), dtype)
+        q = rms_normalised(st.gen, (1, 4, chunk, D), dtype)
+        bt, pt = torch.full((1, L), b, dtype=torch.int64), torch.arange(L)[None]
+        st.cache.insert_kv(0, k.to(DEV), v.to(DEV), input_pos=pt.to(DEV), batch_idx=bt.to(DEV))
+        lim = torch.arange(prefix + 1, L + 1, dtype=torch.int32)
+        pk, pv = st.pool_planes()
+        ws = st.cache.prefill_workspace(chunk, 4, D, 2, dtype)
+        assert ws is not False
+        rb = torch.full((chunk,), b, dtype=torch.int64)
+        out, lse = ops.paged_prefill(q.to(DEV), pk, pv, st.cache.page_table, rb.to(DEV), lim.to(DEV), P,
+                                     workspace=ws, score_bound=1.1 * D ** 0.5)
+        eo, el = O.prefill_attention_paged(f64(q), f64(pk), f64(pv), st.mirror.page_table, rb.numpy(), None, lim.numpy(), P)
+        assert_close(out, lse, eo, el, dtype, lse_atol=BOUNDED_LSE_ATOL)
+
+
+def test_cfg3_chunked_prefill_shape_with_the_score_bound():
+    """BASELINE configs[2] at full size on the bounded path, the bound taken from the norms of the rows."""
+    import bench
+
+    case = bench.make_prefill_case("cfg3", device=DEV)
+    case.append()
+    assert case.score_bound > 0
+    out, lse = case.attend()
+    pk, pv = case.pool_k.float().cpu().numpy(), case.pool_v.float().cpu().numpy()
+    bidx = case.batch_idx.cpu().numpy().reshape(-1)
+    lim = case.row_limit.cpu().numpy()
+    for s in (1, len(case.slots) - 2):
+        rows = np.flatnonzero(bidx == case.slots[s])[3::11]
+        eo, el = O.prefill_attention_paged(f64(case.q[:, :, rows]), pk, pv, case.page_table.cpu().numpy(),
+                                           bidx[rows], None, lim[rows], case.page_size)
+        assert_close(out[:, :, rows], lse[:, :, rows], eo, el, torch.bfloat16, lse_atol=BOUNDED_LSE_ATOL)
