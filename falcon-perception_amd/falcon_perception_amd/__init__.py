@@ -13,7 +13,7 @@ from .paged_attention import PagedKVCache  # noqa: F401
 __all__ = ["KVCacheBase", "PagedKVCache", "attention", "kv_cache", "ops", "paged_attention", "install"]
 
 
-def install(kv_rep: int = 1, qk_norm: bool = False) -> None:
+def install(kv_rep: int = 1, qk_norm: bool = False, fuse_decode_append: bool = True) -> None:
     """Serve the reference's module names from this package.
 
     After `install()`, `import falcon_perception.paged_attention`,
@@ -33,6 +33,12 @@ def install(kv_rep: int = 1, qk_norm: bool = False) -> None:
     embedding, as every variant of the reference does (`model.py:110-116`): |q| = |k| = sqrt(head_dim),
     so the attention scores are bounded and the bf16 prefill kernel runs its softmax without a running
     maximum (`score_bound` of `fp_paged_prefill`).  Leave it off for a model with learned norm weights.
+
+    `fuse_decode_append` (default on): the decode `insert_kv` of the caches created afterwards hands its rows
+    to the attention call that follows it in the reference's model (`model.py:150-162`), which appends and
+    attends in one launch; `PagedKVCache.flush` and every other entry of the cache append them first.  Turn
+    it off for a model that reads the pool views `insert_kv` returns by any other means than the attention
+    callables of this package.
     """
     import sys
 
@@ -40,6 +46,7 @@ def install(kv_rep: int = 1, qk_norm: bool = False) -> None:
         raise ValueError("kv_rep must be at least 1")
     PagedKVCache.default_kv_rep = int(kv_rep)
     PagedKVCache.default_qk_normalised = bool(qk_norm)
+    PagedKVCache.default_fuse_decode_append = bool(fuse_decode_append)
     sys.modules["falcon_perception.kv_cache"] = kv_cache
     sys.modules["falcon_perception.paged_attention"] = paged_attention
     sys.modules["falcon_perception.attention"] = attention

@@ -114,7 +114,7 @@ class HybridPrefillMask:
     """
 
     def __init__(self, cache, batch_idx: Tensor, input_ids: Tensor, soi_id: int, eoi_id: int, block_size: int,
-                 open_spans=None, validate: bool = True, row_hi: Tensor | None = None):
+                 open_spans=None, validate: bool | str = "deferred", row_hi: Tensor | None = None):
         self.cache = cache
         self.batch_idx = batch_idx
         self.input_ids = input_ids
@@ -131,16 +131,18 @@ class HybridPrefillMask:
         self._step_layer = -1  # layer that asked last: a layer id that does not grow starts a new step
         self._row_limit = None
 
-    def _limits_from_ids(self, open_spans, validate: bool) -> Tensor:
-        """Run the row-limit kernel; reject packed rows whose hybrid mask is not one limit per row.
+    def _limits_from_ids(self, open_spans, validate) -> Tensor:
+        """Run the row-limit kernel and hand its report to the cache.
 
         The reference's `or_masks(image_prefix, document_causal)` (`paged_attention.py:350-361`) counts
         soi / eoi tokens over the whole packed row.  A span that is still open where the document changes
         would let its rows see the next document, and a chunk that starts inside a span has no soi to
-        count: neither occurs in the reference's engine (whole sequences, `paged_inference.py:637-672`),
-        and both are refused here instead of being answered with a causal mask.  `open_spans` (cache
-        slots) declares the second case, which is then served: those rows are bidirectional up to the eoi.
-        Reading the kernel's status word waits for the stream once per prefill step."""
+        count: neither occurs in the reference's engine (whole sequences, `paged_inference.py:637-672`).
+        `open_spans` (cache slots) declares the second case, which is then served: those rows are
+        bidirectional up to the eoi.  When and how the kernel's report is looked at is `validate`
+        (`PagedKVCache.create_prefill_blockmask`); only `validate=True` waits for the stream here."""
+        if validate not in (True, False, "deferred"):
+            raise ValueError('validate must be True, False or "deferred"')
         dev = self.batch_idx.device
         open_at_start = None
         if open_spans is not None:
@@ -151,16 +153,12 @@ class HybridPrefillMask:
         status = torch.zeros(1, dtype=torch.int32, device=dev) if validate else None
         row_hi = ops.hybrid_row_limits(self.input_ids, self.soi_id, self.eoi_id, self.batch_idx,
                                        open_at_start, status)
-        if validate:
+        if validate is True:
             bits = int(status.item())
-            if bits & 1:
-                raise RuntimeError(
-                    "create_prefill_blockmask: an end-of-image token closes a span that was not opened in this "
-                    "packed row; a chunk that starts inside an image span must be declared with open_spans=[slot]")
-            if bits & 2:
-                raise RuntimeError(
-                    "create_prefill_blockmask: an image span is still open where batch_idx changes or the packed "
-                    "row ends; its rows would need keys of another sequence or keys that are not cached yet")
+            if bits:
+                self.cache._report_mask_status(bits, late=False)
+        elif validate == "deferred":
+            self.cache._defer_mask_status(status)
         return row_hi
 
     def row_limit(self, input_pos: Tensor, layer_id: int = 0) -> Tensor:
@@ -243,11 +241,23 @@ def compiled_flex_attn_decode(q: Tensor, k: Tensor, v: Tensor, score_mod=None, b
     workspace, split_tokens = cache.decode_launch(q.shape[0], q.shape[1], q.shape[3], block_mask.max_context, wg_heads)
     # the pool views insert_kv returned, as planes [H, N, D]: the cache keeps both forms of every layer
     pools = cache._pools[step.layer_id]
-    pool_k, pool_v = cache._planes[step.layer_id] if (k is pools[0] and v is pools[1]) else (k[0], v[0])
+    own = k is pools[0] and v is pools[1]
+    pool_k, pool_v = cache._planes[step.layer_id] if own else (k[0], v[0])
+    k_new = v_new = None
+    if step.k_new is not None:
+        # the append of this step was left to this launch (`PagedKVCache.fuse_decode_append`): the kernel
+        # appends the rows and attends over them.  Any other k, v than the pool views of the step's layer
+        # means the caller is not the model's insert -> attend pair, and the plain append runs first.
+        if own and step.k_new.shape[0] == q.shape[0]:
+            k_new, v_new = step.k_new, step.v_new
+            cache.last_decode_step = step._replace(k_new=None, v_new=None)
+        else:
+            cache.flush()
     out, lse = ops.paged_decode(
         q, pool_k, pool_v, cache.page_table, block_mask.batch_idx, step.input_pos,
         cache.page_size, block_mask.max_context, scale=scale,
         workspace=workspace, split_tokens=split_tokens, sinks=sinks, kv_rep=kv_rep,
+        k_new=k_new, v_new=v_new,
     )
     return _result(out, lse, return_aux, return_lse)
 
@@ -272,6 +282,7 @@ def compiled_flex_attn_prefill(q: Tensor, k: Tensor, v: Tensor, score_mod=None, 
     if score_mod is not None:
         raise RuntimeError("score_mod is not supported on the paged prefill path")
     cache = block_mask.cache
+    cache.flush()
     step = cache.last_prefill_step
     if step is None:
         raise RuntimeError("paged prefill attention called before PagedKVCache.insert_kv for this step")

@@ -10,6 +10,7 @@ operation on K/V data (append, block-id lookup) is a HIP kernel reached through
 
 from __future__ import annotations
 
+import warnings
 from typing import NamedTuple
 
 import torch
@@ -26,11 +27,14 @@ def _cdiv(x, multiple) -> int:
 
 
 class StepMeta(NamedTuple):
-    """What `insert_kv` saw last: the attention call of the same layer reads it."""
+    """What `insert_kv` saw last: the attention call of the same layer reads it.  `k_new` / `v_new` are the
+    rows of a decode step whose append has been left to the attention launch (`fuse_decode_append`)."""
 
     layer_id: int
     input_pos: Tensor
     batch_idx: Tensor
+    k_new: Tensor | None = None
+    v_new: Tensor | None = None
 
 
 class PagedKVCache(KVCacheBase):
@@ -52,12 +56,15 @@ class PagedKVCache(KVCacheBase):
     table (`get_mask_mod`, the element mask of the reference's flex kernels) is then unavailable.
     """
 
-    default_kv_rep = 1  # kv_rep of caches created from now on, see `falcon_perception_amd.install`
-    default_qk_normalised = False  # likewise: whether the q and k rows the model produces have norm sqrt(head_dim)
+    # what `falcon_perception_amd.install` sets for the caches an unedited engine creates afterwards
+    default_kv_rep = 1
+    default_qk_normalised = False
+    default_fuse_decode_append = False
 
     def __init__(self, n_pages: int, page_size: int, max_batch_size: int, n_heads: int, head_dim: int,
                  num_layers: int, dtype: torch.dtype, device: str | torch.device = "cuda",
-                 max_blocks_per_seq: int | None = None):
+                 max_blocks_per_seq: int | None = None, *, kv_rep: int | None = None,
+                 qk_normalised: bool | None = None, fuse_decode_append: bool | None = None):
         self.n_pages = n_pages
         self.page_size = page_size
         self.max_batch_size = max_batch_size
@@ -78,30 +85,65 @@ class PagedKVCache(KVCacheBase):
         self.free_batch_idx: list[int] = list(range(max_batch_size - 1, 0, -1))
 
         self.kv_shape = (num_layers, 2, 1, n_heads, n_pages * page_size, head_dim)
-        self.kv_cache = torch.zeros(self.kv_shape, dtype=dtype, device=device)
+        self._kv = torch.zeros(self.kv_shape, dtype=dtype, device=device)  # `kv_cache`, see the property
         # views of every layer's K and V planes, made once: [H, N, D] for the kernels, [1, H, N, D] as returned
         # to the model (an indexing operation per layer and call costs the host more than the launch itself)
-        self._planes = [(self.kv_cache[l, 0, 0], self.kv_cache[l, 1, 0]) for l in range(num_layers)]
-        self._pools = [(self.kv_cache[l, 0], self.kv_cache[l, 1]) for l in range(num_layers)]
+        self._planes = [(self._kv[l, 0, 0], self._kv[l, 1, 0]) for l in range(num_layers)]
+        self._pools = [(self._kv[l, 0], self._kv[l, 1]) for l in range(num_layers)]
 
         # 1, or n_heads // n_kv_heads when the cached V heads are plain copies inside a group (the model's
-        # repeat_kv, model.py:112-113): the decode kernel then reads V once per group.  Taken from the class
-        # default (`falcon_perception_amd.install(kv_rep=...)` sets it for an engine that is not edited) when
-        # it divides this cache's head count.
-        self.kv_rep = self.default_kv_rep if n_heads % self.default_kv_rep == 0 else 1
+        # repeat_kv, model.py:112-113): the decode kernel then reads V once per group.  An argument of this
+        # constructor, or else the class default (`falcon_perception_amd.install(kv_rep=...)` sets it for an
+        # engine that is not edited) when it divides this cache's head count.  A value that came from the
+        # class default is checked against the V rows of the first prefill step (`_check_v_copies`).
+        if kv_rep is None:
+            self.kv_rep = self.default_kv_rep if n_heads % self.default_kv_rep == 0 else 1
+            self._kv_rep_unverified = self.kv_rep > 1
+        else:
+            if kv_rep < 1 or n_heads % kv_rep:
+                raise ValueError(f"kv_rep={kv_rep} must divide the {n_heads} cached heads")
+            self.kv_rep = int(kv_rep)
+            self._kv_rep_unverified = False
         # Whether every q and k row has norm sqrt(head_dim): the reference's model RMS-normalises both without a
         # weight and rotates them (model.py:110-116).  |scale * q.k| is then at most scale * head_dim, and the
         # bf16 prefill kernel runs its softmax without a running maximum (`score_bound`).  Set by
         # `insert_qkv_norm_rope`, which does the normalisation itself, or by `install(qk_norm=True)`.
-        self.qk_normalised = self.default_qk_normalised
+        self.qk_normalised = self.default_qk_normalised if qk_normalised is None else bool(qk_normalised)
+        # Whether a decode `insert_kv` leaves its rows to the attention launch of the same layer, which then
+        # appends and attends in one kernel (`fp_paged_decode_append`).  The reference's model calls the two
+        # back to back (model.py:150-162) and nothing reads the pool in between; whatever else touches the
+        # cache first (`flush`, another insert, `kv_cache`, erase, a prefill mask) launches the plain append.
+        self.fuse_decode_append = (self.default_fuse_decode_append if fuse_decode_append is None
+                                   else bool(fuse_decode_append))
 
         # what the attention callables need from the step in flight
         self.last_decode_step: StepMeta | None = None
         self.last_prefill_step: StepMeta | None = None
         self._workspace: Tensor | None = None
+        self._retired_workspaces: list[Tensor] = []  # graphs captured earlier still write to these
         self._decode_launch: dict[tuple, tuple[int, int]] = {}
         self._prefill_workspace: Tensor | None = None
         self._prefill_need: dict[tuple, int] = {}
+        # status word of the last prefill mask, on its way to the host (`check_prefill_masks`)
+        self._mask_status_host: Tensor | None = None
+        self._mask_status_event = None
+
+    @property
+    def kv_cache(self) -> Tensor:
+        """The pool [L, 2, 1, H, n_pages * page_size, D] (`paged_attention.py:73-74`).  Reading it first
+        launches an append that is still waiting for its attention call."""
+        self.flush()
+        return self._kv
+
+    def flush(self) -> None:
+        """Launch the append of a decode step whose rows were left to the attention call (no-op otherwise)."""
+        step = self.last_decode_step
+        if step is None or step.k_new is None:
+            return
+        self.last_decode_step = step._replace(k_new=None, v_new=None)
+        pool_k, pool_v = self._planes[step.layer_id]
+        ops.kv_append(pool_k, pool_v, step.k_new, step.v_new, self.page_table, step.batch_idx, step.input_pos,
+                      self.page_size, clamp_negative=True)
 
     # ------------------------------------------------------------------ append
     def insert_kv(self, layer_id: int, k: Tensor, v: Tensor, input_pos: Tensor | None = None,
@@ -111,6 +153,7 @@ class PagedKVCache(KVCacheBase):
         assert input_pos is not None, "input_pos is required for paged kv cache"
         assert batch_idx is not None, "batch_idx is required for paged kv cache"
         assert batch_idx.ndim in [1, 2], "batch_idx must be 1D (decode) or 2D (prefill 1xL)"
+        self.flush()
         if batch_idx.ndim == 1:
             return self.assign(layer_id, batch_idx, input_pos, k, v)
         return self.assign_prefill_no_paging(layer_id, k, v, input_pos, batch_idx)
@@ -120,12 +163,17 @@ class PagedKVCache(KVCacheBase):
         (batch_idx[b], input_pos[b, s]); unmapped (-1) pages are redirected to the
         reserved page 0.  Returns the layer's whole K and V pools, [1, H, N, D] views."""
         B, H, S, K_D = k_val.shape
-        _, _, _, H_cache, MAX_S, D_cache = self.kv_cache.shape
+        _, _, _, H_cache, MAX_S, D_cache = self.kv_shape
         assert H_cache == H, "number of heads must match"
         assert MAX_S >= S, "cache must have enough space"
         assert D_cache == K_D, "hidden dim must match"
         assert input_pos.shape == (B, S), "input_pos must have the same shape as val"
         assert batch_idx.shape == (B,), "batch_idx must have one dimension only"
+        self.flush()
+        if self.fuse_decode_append and S == 1 and k_val.dtype == self.dtype and v_val.dtype == self.dtype:
+            # the attention call of this layer appends the rows itself (compiled_flex_attn_decode)
+            self.last_decode_step = StepMeta(layer_id, input_pos, batch_idx, k_val, v_val)
+            return self._pools[layer_id]
         pool_k, pool_v = self._planes[layer_id]
         ops.kv_append(pool_k, pool_v, k_val, v_val, self.page_table, batch_idx, input_pos, self.page_size,
                       clamp_negative=True)
@@ -142,6 +190,9 @@ class PagedKVCache(KVCacheBase):
         assert input_pos.ndim == 2, "input_pos must be a 2D tensor"
         assert k_val.ndim == 4, "k_val must be a 4D tensor"
         assert v_val.ndim == 4, "v_val must be a 4D tensor"
+        self.flush()
+        if self._kv_rep_unverified:
+            self._check_v_copies(v_val)
         pool_k, pool_v = self._planes[layer_id]
         # [1, H, L, D] seen as L row groups of one token each: the strides say so, no views are made
         ops.kv_append(pool_k, pool_v, k_val, v_val, self.page_table, batch_idx, input_pos, self.page_size,
@@ -161,6 +212,7 @@ class PagedKVCache(KVCacheBase):
         attention does not read."""
         decode = batch_idx.ndim == 1
         assert batch_idx.ndim in [1, 2], "batch_idx must be 1D (decode) or 2D (prefill 1xL)"
+        self.flush()
         B, S = xq.shape[0], xq.shape[1]
         assert input_pos.shape == (B, S), "input_pos must be [B, S]"
         if decode:
@@ -175,6 +227,20 @@ class PagedKVCache(KVCacheBase):
         else:
             self.last_prefill_step = StepMeta(layer_id, input_pos, batch_idx)
         return (q, *self._pools[layer_id])
+
+    def _check_v_copies(self, v_val: Tensor) -> None:
+        """`kv_rep` > 1 that came from the class default, not from this cache's creator, is a claim about a
+        model this cache may not belong to (a second engine in the process, a model without head repeat):
+        the V rows of the first prefill step are compared inside each group, once, and a cache whose heads
+        differ refuses to go on instead of decoding through the shared-V read (one wait for the stream)."""
+        self._kv_rep_unverified = False
+        H = v_val.shape[1]
+        groups = v_val.reshape(v_val.shape[0], H // self.kv_rep, self.kv_rep, *v_val.shape[2:])
+        if not bool((groups == groups[:, :, :1]).all()):
+            raise RuntimeError(
+                f"this cache took kv_rep={self.kv_rep} from install(kv_rep=...), but the V heads it is given are not "
+                f"{self.kv_rep} identical copies per group; create it with PagedKVCache(..., kv_rep=1) or call "
+                "install(kv_rep=1) before the engine that owns it is built")
 
     def v_copies_are_identical(self, layer_id: int = 0) -> bool:
         """Whether the V plane of a layer really holds `kv_rep` identical heads per group (bit for bit, over
@@ -218,20 +284,21 @@ class PagedKVCache(KVCacheBase):
             return True
         n_new = _cdiv(seq_len - have, self.page_size)
         fits = bool(n_new <= self.num_free_pages)
-        if have // self.page_size + n_new > self.table_cols:  # only a sparse table can be narrower than the pool
-            if dry_run:
-                return False
-            raise RuntimeError(
-                f"Cannot reserve a sequence of length {seq_len} in batch {batch_idx_int}: "
-                f"the page table holds {self.table_cols} blocks of {self.page_size} tokens per sequence."
-            )
+        # a table narrower than the pool (max_blocks_per_seq) can be full while pages are free; with the
+        # reference's dense table the pool always runs out first and its message is the one raised
+        in_table = have // self.page_size + n_new <= self.table_cols
         if dry_run:
-            return fits
+            return fits and in_table
         if not fits:
             raise RuntimeError(
                 f"Cannot reserve {n_new} pages for a sequence of length {seq_len} "
                 f"in batch {batch_idx_int}. Only {self.num_free_pages} pages available. "
                 f"Current capacity is {have} tokens."
+            )
+        if not in_table:
+            raise RuntimeError(
+                f"Cannot reserve a sequence of length {seq_len} in batch {batch_idx_int}: "
+                f"the page table holds {self.table_cols} blocks of {self.page_size} tokens per sequence."
             )
         first = have // self.page_size
         pages = self.free_pages[-n_new:]
@@ -247,6 +314,8 @@ class PagedKVCache(KVCacheBase):
 
     def erase(self, batch_idx: int) -> None:
         """Release a slot and its pages; table rows go back to -1, pool bytes stay (:166-182)."""
+        self.flush()
+        self.check_prefill_masks(wait=False)
         self.free_batch_idx.append(batch_idx)
         self.free_pages.extend(reversed(self.page_table_cpu[batch_idx]))
         self.page_table_cpu[batch_idx] = []
@@ -320,16 +389,71 @@ class PagedKVCache(KVCacheBase):
         )
 
     def create_prefill_blockmask(self, batch_idx: Tensor, input_ids: Tensor, soi_id: int, eoi_id: int,
-                                 BLOCK_SIZE: int = 128, *, open_spans=None, validate: bool = True) -> HybridPrefillMask:
+                                 BLOCK_SIZE: int = 128, *, open_spans=None,
+                                 validate: bool | str = "deferred") -> HybridPrefillMask:
         """Mask of a packed prefill step: document-causal OR image-prefix (:343-362).
 
-        `open_spans` and `validate` are not arguments of the reference: `open_spans` lists the cache slots
-        whose chunk begins inside an image span that an earlier chunk opened; with `validate` (default) a
-        packed row whose spans cross a document boundary, the end of the row, or start before it undeclared
-        raises RuntimeError (one host read of a device word) instead of yielding a wrong mask."""
+        `open_spans` and `validate` are not arguments of the reference.  `open_spans` lists the cache slots
+        whose chunk begins inside an image span that an earlier chunk opened.  The row-limit kernel reports
+        packed rows for which one limit per row is not the reference's mask (an end-of-image token with no
+        span open; a span still open where the document changes or the row ends), and `validate` says when
+        the host looks at that report:
+          "deferred" (default)  the word travels to pinned host memory behind the kernel and is looked at by
+                     the next `create_prefill_blockmask`, `erase` or `check_prefill_masks` -- no wait in this
+                     call, as the reference's mask construction has none (its engine waits once per step,
+                     `paged_inference.py:1083`).  A span open across a boundary then raises RuntimeError one
+                     step late; a stray end-of-image token only warns, because the limits the kernel wrote for
+                     it are the reference's own mask (which counts delimiters over the whole packed row,
+                     `attention.py:75-96`) unless the caller is prefilling in chunks;
+          True       this call waits for the kernel and raises for either report: for callers that prefill in
+                     chunks (an undeclared chunk start inside a span) and for tests;
+          False      nobody looks."""
         assert batch_idx.ndim == 2 and batch_idx.shape[0] == 1
+        self.flush()
+        self.check_prefill_masks(wait=True)  # the report of the step before: landed long ago
         return HybridPrefillMask(self, batch_idx, input_ids, soi_id, eoi_id, BLOCK_SIZE,
                                  open_spans=open_spans, validate=validate)
+
+    _MASK_REPORTS = (
+        "an end-of-image token closes a span that was not opened in this packed row; a chunk that starts inside "
+        "an image span must be declared with open_spans=[slot]",
+        "an image span is still open where batch_idx changes or the packed row ends; its rows would need keys of "
+        "another sequence or keys that are not cached yet",
+    )
+
+    def _report_mask_status(self, bits: int, late: bool) -> None:
+        when = "the previous create_prefill_blockmask" if late else "create_prefill_blockmask"
+        if bits & 2:
+            raise RuntimeError(f"{when}: {self._MASK_REPORTS[1]}")
+        if bits & 1:
+            if not late:
+                raise RuntimeError(f"{when}: {self._MASK_REPORTS[0]}")
+            warnings.warn(f"{when}: {self._MASK_REPORTS[0]} (the rows were masked as the reference masks them: "
+                          "delimiters counted over the whole packed row)", RuntimeWarning, stacklevel=3)
+
+    def _defer_mask_status(self, status: Tensor) -> None:
+        """Send the status word of a row-limit launch to pinned host memory behind the kernel."""
+        if self._mask_status_host is None:
+            self._mask_status_host = torch.zeros(1, dtype=torch.int32, pin_memory=True)
+            self._mask_status_event = torch.cuda.Event()
+        self._mask_status_host.copy_(status, non_blocking=True)
+        self._mask_status_event.record(torch.cuda.current_stream(status.device))
+        self._mask_status_pending = True
+
+    _mask_status_pending = False
+
+    def check_prefill_masks(self, wait: bool = True) -> None:
+        """Look at the report of the last deferred `create_prefill_blockmask` (see there).  `wait=False` looks
+        only if the word has already arrived.  An engine calls this where it waits for the device anyway."""
+        if not self._mask_status_pending:
+            return
+        if not wait and not self._mask_status_event.query():
+            return
+        self._mask_status_event.synchronize()
+        self._mask_status_pending = False
+        bits = int(self._mask_status_host[0])
+        if bits:
+            self._report_mask_status(bits, late=True)
 
     # ------------------------------------------------ decode launch parameters
     def decode_split_tokens(self, B: int, Hc: int, max_context: int) -> int:
@@ -350,12 +474,19 @@ class PagedKVCache(KVCacheBase):
         key = (B, Hq, D, max_context, Hc)
         hit = self._decode_launch.get(key)
         if hit is None:
+            # sized for the largest batch and the longest context the page table can hold, at the finest split
+            # either can get, so that later shapes fit.  Should one not (more query heads), the old buffer is
+            # kept alive: graphs captured with it go on writing to it.
             worst_b = max(B, self.max_batch_size)
-            finest = min(self.decode_split_tokens(1, Hc, max_context),
-                         self.decode_split_tokens(worst_b, Hc, max_context))
-            need = ops.decode_workspace_bytes(worst_b, Hq, D, max_context, finest)
+            worst_ctx = max(max_context, self.table_cols * self.page_size)
+            need = 0
+            for ctx in {max_context, worst_ctx}:
+                finest = min(self.decode_split_tokens(1, Hc, ctx), self.decode_split_tokens(worst_b, Hc, ctx))
+                need = max(need, ops.decode_workspace_bytes(worst_b, Hq, D, ctx, finest))
             if need and (self._workspace is None or self._workspace.numel() < need):
-                self._workspace = torch.empty(need, dtype=torch.uint8, device=self.kv_cache.device)
+                if self._workspace is not None:
+                    self._retired_workspaces.append(self._workspace)
+                self._workspace = torch.empty(need, dtype=torch.uint8, device=self._kv.device)
             hit = (need, self.decode_split_tokens(B, Hc, max_context))
             self._decode_launch[key] = hit
         return (self._workspace if hit[0] else None), hit[1]
@@ -377,5 +508,5 @@ class PagedKVCache(KVCacheBase):
         if need == 0:
             return False
         if self._prefill_workspace is None or self._prefill_workspace.numel() < need:
-            self._prefill_workspace = torch.empty(need, dtype=torch.uint8, device=self.kv_cache.device)
+            self._prefill_workspace = torch.empty(need, dtype=torch.uint8, device=self._kv.device)
         return self._prefill_workspace

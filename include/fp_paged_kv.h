@@ -332,11 +332,18 @@ int fp_qkv_norm_rope_append(const void* xq, const void* xk, const void* xv,
  *             paged_inference.py:637-672); the rows up to the span's eoi then get the eoi's index
  *   row_hi    [L] int32 out: packed index one past the last key row q may see
  *             = max(q + 1, end of q's image span)
- *   status    NULL, or one int32 out (written, not accumulated): 0 when row_hi is the reference's
- *             mask; bit 0 = an eoi with no span open (a chunk that starts inside a span and was not
- *             declared); bit 1 = a span still open where batch_idx changes or the row ends (its
- *             rows would need keys of another document or keys not yet cached).  row_hi is then
- *             not a usable mask and the caller must reject the step.
+ *   status    NULL, or one int32 out (written, not accumulated): 0 when row_hi is the mask of a packed
+ *             row of whole sequences.  Delimiters are counted over the WHOLE packed row, as the
+ *             reference's mask counts them (attention.py:77-79), not per document:
+ *             bit 0 = at some token more eoi than soi (virtual ones included) have been seen: an eoi
+ *             with no span open.  row_hi is then still what the reference's predicate gives for this
+ *             row (nothing is inside a span while the balance is not positive), which is the right
+ *             mask for a stray eoi and the wrong one for a chunk that starts inside a span and was
+ *             not declared;
+ *             bit 1 = the balance is positive where batch_idx changes or the row ends: a span still
+ *             open there (its rows would need keys of another document or keys not yet cached).
+ *             row_hi is then not a usable mask and the caller must reject the step.  An eoi of the
+ *             NEXT document closes such a span in the global count, so bit 0 is not raised with it.
  * L <= 65536 (one workgroup scans the row).
  */
 int fp_hybrid_row_limits(const int64_t* input_ids, const int64_t* batch_idx,

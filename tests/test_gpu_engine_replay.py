@@ -28,8 +28,9 @@ ATOL, RTOL = 2e-2, 1e-2
 class MiniEngine:
     """The parts of PagedInferenceEngine that touch the cache, with random K/V/Q instead of a model."""
 
-    def __init__(self):
-        self.cache = PagedKVCache(N_PAGES, P, MAX_BS, H, D, LAYERS, DTYPE, device=DEV)
+    def __init__(self, fuse_decode_append=False):
+        self.cache = PagedKVCache(N_PAGES, P, MAX_BS, H, D, LAYERS, DTYPE, device=DEV,
+                                  fuse_decode_append=fuse_decode_append)
         self.block_mask = self.cache.create_causal_blockmask(B=MAX_BS, L=MAX_SEQ)
         self.input_pos = torch.zeros(MAX_BS, dtype=torch.int32, device=DEV)
         self.gen = torch.Generator().manual_seed(0)
@@ -59,6 +60,7 @@ class MiniEngine:
             K, V = self.cache.insert_kv(layer, k[layer, :B], v[layer, :B], input_pos=pos.view(B, 1), batch_idx=batch_idx)
             o, aux = A.compiled_flex_attn_decode(q[layer, :B], K, V, block_mask=mask, return_aux=AuxRequest(lse=True),
                                                  kernel_options={})
+            assert self.cache.last_decode_step.k_new is None  # the rows are in the pool, by either route
             out[layer, :B] = o
             lse[layer, :B] = aux.lse
 
@@ -180,11 +182,67 @@ def tokens(n_text_before, n_img, n_text_after):
     return [TXT] * n_text_before + img + [TXT] * n_text_after
 
 
-def test_engine_call_sequence():
-    eng = MiniEngine()
+@pytest.mark.parametrize("fuse_decode_append", [False, True], ids=["append-launch", "append-in-attention"])
+def test_engine_call_sequence(fuse_decode_append):
+    """`fuse_decode_append` is what `install()` switches on for an engine that is not edited: the decode
+    `insert_kv` launches nothing and the attention call that follows appends and attends in one kernel.  The
+    pool is compared with the oracle's after the attention calls either way."""
+    eng = MiniEngine(fuse_decode_append)
     eng.capture()
     with torch.inference_mode():
         generate(eng)
+
+
+def test_a_decode_append_left_to_the_attention_call_is_launched_by_whatever_comes_first():
+    """With `fuse_decode_append` the rows of a decode `insert_kv` wait for the attention call.  Reading
+    `kv_cache`, another insert, `erase` or `flush` must find them in the pool."""
+    cache = PagedKVCache(8, P, 4, H, D, 2, DTYPE, device=DEV, fuse_decode_append=True)
+    slot = cache.allocate()
+    cache.reserve(slot, torch.tensor([slot], device=DEV), 3 * P)
+    gen = torch.Generator().manual_seed(5)
+    bidx = torch.tensor([slot], device=DEV)
+    page = cache.page_table_cpu[slot][0]
+
+    def row(layer, pos):
+        return cache.kv_cache[layer, 0, 0, :, page * P + pos].clone()
+
+    k, v = (randn(gen, (1, H, 1, D), DTYPE).to(DEV) for _ in range(2))
+    cache.insert_kv(0, k, v, input_pos=torch.tensor([[2]], dtype=torch.int32, device=DEV), batch_idx=bidx)
+    assert cache.last_decode_step.k_new is k  # nothing launched yet
+    assert torch.equal(row(0, 2), k[0, :, 0])  # the property launches the append
+    assert cache.last_decode_step.k_new is None
+    k2, v2 = (randn(gen, (1, H, 1, D), DTYPE).to(DEV) for _ in range(2))
+    cache.insert_kv(0, k2, v2, input_pos=torch.tensor([[3]], dtype=torch.int32, device=DEV), batch_idx=bidx)
+    cache.insert_kv(1, k, v, input_pos=torch.tensor([[3]], dtype=torch.int32, device=DEV), batch_idx=bidx)  # next layer first
+    assert torch.equal(cache._kv[0, 0, 0, :, page * P + 3], k2[0, :, 0])
+    cache.flush()
+    assert torch.equal(cache._kv[1, 1, 0, :, page * P + 3], v[0, :, 0])
+    cache.insert_kv(0, k2, v2, input_pos=torch.tensor([[4]], dtype=torch.int32, device=DEV), batch_idx=bidx)
+    cache.erase(slot)  # the rows land before the slot's pages go back
+    assert torch.equal(cache._kv[0, 0, 0, :, page * P + 4], k2[0, :, 0])
+
+
+def test_kv_rep_from_install_is_checked_against_the_first_prefill(monkeypatch):
+    """A cache that took kv_rep from the class default (install(kv_rep=2)) and is then fed V heads that are not
+    copies -- a second engine in the process, a model without head repeat -- refuses at its first prefill."""
+    monkeypatch.setattr(PagedKVCache, "default_kv_rep", 2)
+    gen = torch.Generator().manual_seed(6)
+    t = lambda a: torch.tensor([a], device=DEV)
+    for copies in (True, False):
+        cache = PagedKVCache(8, P, 4, H, D, 1, DTYPE, device=DEV)
+        assert cache.kv_rep == 2
+        slot = cache.allocate()
+        cache.reserve(slot, torch.tensor([slot], device=DEV), 10)
+        k = randn(gen, (1, H, 10, D), DTYPE).to(DEV)
+        v = randn(gen, (1, H // 2, 10, D), DTYPE).to(DEV).repeat_interleave(2, dim=1) if copies else randn(gen, (1, H, 10, D), DTYPE).to(DEV)
+        if copies:
+            cache.insert_kv(0, k, v, input_pos=t(list(range(10))), batch_idx=t([slot] * 10))
+            assert cache.v_copies_are_identical()
+        else:
+            with pytest.raises(RuntimeError, match="not 2 identical copies"):
+                cache.insert_kv(0, k, v, input_pos=t(list(range(10))), batch_idx=t([slot] * 10))
+    explicit = PagedKVCache(8, P, 4, H, D, 1, DTYPE, device=DEV, kv_rep=1)
+    assert explicit.kv_rep == 1 and not explicit._kv_rep_unverified
 
 
 def generate(eng):

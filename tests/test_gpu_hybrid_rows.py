@@ -86,3 +86,16 @@ def test_status_on_long_rows():
     ids[4990] = SOI  # and where the row ends
     ids[3990] = TXT
     assert limits_with_status(ids, bidx, [2])[1] == 2
+
+
+def test_status_of_a_span_open_across_a_document_boundary():
+    """Where the kernel's status and the oracle's differ: a span left open by document 1 and an eoi in document 2.
+    The kernel counts delimiters over the whole packed row, as the reference's mask does (attention.py:75-96), so
+    the second document's eoi closes the first document's span and no balance ever drops below zero: status 2.
+    The oracle walks every document with its own balance and also sees an eoi with no span open: status 3.  Bit 1
+    is set by both, and bit 1 alone rejects the step."""
+    ids = np.array([TXT] * 3 + [SOI] + [IMG] * 20 + [TXT] * 8 + [EOI] + [TXT] * 4)
+    bidx = np.array([1] * 24 + [2] * 13)
+    _, status = limits_with_status(ids, bidx, [])
+    _, es = O.chunk_row_limits(bidx, ids, SOI, EOI)
+    assert status == 2 and es == 3 and (status & es & 2)

@@ -231,12 +231,12 @@ def test_chunk_boundary_inside_the_image_span(cut):
     dev = lambda a: torch.from_numpy(a)[None].to(DEV)
     if cut > 12:
         with pytest.raises(RuntimeError, match="still open"):
-            cache.create_prefill_blockmask(dev(bidx[:cut]), dev(ids[:cut]), SOI, EOI)
+            cache.create_prefill_blockmask(dev(bidx[:cut]), dev(ids[:cut]), SOI, EOI, validate=True)
     cache.insert_kv(0, k[:, :, :cut].to(DEV), v[:, :, :cut].to(DEV), input_pos=dev(pos[:cut]), batch_idx=dev(bidx[:cut]))
     if 12 < cut <= 212:
         with pytest.raises(RuntimeError, match="open_spans"):
-            cache.create_prefill_blockmask(dev(bidx[cut:]), dev(ids[cut:]), SOI, EOI)
-    mask = cache.create_prefill_blockmask(dev(bidx[cut:]), dev(ids[cut:]), SOI, EOI, open_spans=[b])
+            cache.create_prefill_blockmask(dev(bidx[cut:]), dev(ids[cut:]), SOI, EOI, validate=True)
+    mask = cache.create_prefill_blockmask(dev(bidx[cut:]), dev(ids[cut:]), SOI, EOI, open_spans=[b], validate=True)
     K, V = cache.insert_kv(0, k[:, :, cut:].to(DEV), v[:, :, cut:].to(DEV), input_pos=dev(pos[cut:]),
                            batch_idx=dev(bidx[cut:]))
     out, aux = A.compiled_flex_attn_prefill(q[:, :, cut:].to(DEV), K, V, block_mask=mask, return_aux=AuxRequest(lse=True))
@@ -250,9 +250,45 @@ def test_span_open_across_a_document_boundary_is_refused():
     st = PagedState(22, n_pages=8, page_size=16, max_batch=4, Hc=1, D=64, dtype=torch.bfloat16)
     dev = lambda a: torch.from_numpy(a)[None].to(DEV)
     with pytest.raises(RuntimeError, match="still open"):
-        st.cache.create_prefill_blockmask(dev(bidx), dev(ids), SOI, EOI)
+        st.cache.create_prefill_blockmask(dev(bidx), dev(ids), SOI, EOI, validate=True)
     # unchecked, the call returns as before (the mask of such a row is unspecified)
     st.cache.create_prefill_blockmask(dev(bidx), dev(ids), SOI, EOI, validate=False)
+    # by default the report travels to the host behind the kernel and the next look at it raises
+    st.cache.create_prefill_blockmask(dev(bidx), dev(ids), SOI, EOI)
+    with pytest.raises(RuntimeError, match="previous create_prefill_blockmask.*still open"):
+        st.cache.check_prefill_masks()
+    st.cache.check_prefill_masks()  # looked at once
+    st.cache.create_prefill_blockmask(dev(bidx), dev(ids), SOI, EOI)
+    with pytest.raises(RuntimeError, match="still open"):
+        st.cache.create_prefill_blockmask(dev(bidx[:20]), dev(ids[:20] * 0 + TXT), SOI, EOI)
+
+
+def test_a_stray_end_of_image_token_is_masked_as_the_reference_masks_it_and_warns_late():
+    """A sequence that sampled an end-of-image token of its own and is prefilled again after a preemption
+    (paged_inference.py:1231-1237) carries an eoi with no span open.  The reference counts delimiters over the
+    whole packed row (attention.py:75-96): nothing is inside a span while closed >= opened, so the stray token
+    and the rows after it are causal -- and so is a LATER image span of the row, whose soi only brings the
+    balance back to zero.  The kernel's limits are that mask; the default call does not wait and the report
+    surfaces as a warning at the next look."""
+    dtype, Hc, G, D, Pg = torch.bfloat16, 1, 2, 64, 16
+    ids = np.array([TXT] * 5 + [EOI] + [TXT] * 6 + [SOI] + [IMG] * 10 + [EOI] + [TXT] * 7)
+    L = len(ids)
+    st = PagedState(23, n_pages=8, page_size=Pg, max_batch=3, Hc=Hc, D=D, dtype=dtype)
+    b = st.add_sequence(L)
+    bidx, pos = np.full(L, b), np.arange(L)
+    dev = lambda a: torch.from_numpy(a)[None].to(DEV)
+    with pytest.raises(RuntimeError, match="open_spans"):
+        st.cache.create_prefill_blockmask(dev(bidx), dev(ids), SOI, EOI, validate=True)
+    mask = st.cache.create_prefill_blockmask(dev(bidx), dev(ids), SOI, EOI)
+    k, v, q = (randn(st.gen, (1, h, L, D), dtype) for h in (Hc, Hc, Hc * G))
+    K, V = st.cache.insert_kv(0, k.to(DEV), v.to(DEV), input_pos=dev(pos), batch_idx=dev(bidx))
+    out, aux = A.compiled_flex_attn_prefill(q.to(DEV), K, V, block_mask=mask, return_aux=AuxRequest(lse=True))
+    # the reference's predicate on a dense grid (oracle: attention.py:75-96 OR document-causal)
+    eo, el = O.prefill_attention_packed(f64(q), f64(k), f64(v), bidx[None], ids[None], SOI, EOI)
+    assert_close(out, aux.lse, eo, el, dtype)
+    assert (mask.row_hi.cpu().numpy() == np.arange(1, L + 1)).all()  # every row causal, the later span included
+    with pytest.warns(RuntimeWarning, match="end-of-image"):
+        st.cache.check_prefill_masks()
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=str)

@@ -237,6 +237,14 @@ def test_mask_mod_factories_match_the_oracle_tables():
     assert A.offset_mask_mod(A.get_causal_mask_mod(), 3)(0, 0, torch.tensor(1), torch.tensor(4)).item()
 
 
+@pytest.fixture(autouse=True)
+def restore_install_defaults(monkeypatch):
+    """`install()` writes class-wide defaults; every test starts from the bare ones and leaves them so."""
+    monkeypatch.setattr(PagedKVCache, "default_kv_rep", 1)
+    monkeypatch.setattr(PagedKVCache, "default_qk_normalised", False)
+    monkeypatch.setattr(PagedKVCache, "default_fuse_decode_append", False)
+
+
 def test_install_serves_the_reference_module_names():
     saved = {k: sys.modules.get(k) for k in
              ("falcon_perception.kv_cache", "falcon_perception.paged_attention", "falcon_perception.attention")}
@@ -316,6 +324,43 @@ def test_install_serves_the_reference_module_names_and_sets_kv_rep(monkeypatch):
     assert PagedKVCache(8, 4, 4, 3, 8, 1, torch.float32, device="cpu").kv_rep == 1  # 3 heads: no groups of 2
     with pytest.raises(ValueError):
         fpa.install(kv_rep=0)
+    # the constructor's own argument wins over the class default and is validated
+    assert PagedKVCache(8, 4, 4, 16, 8, 1, torch.float32, device="cpu", kv_rep=1).kv_rep == 1
+    with pytest.raises(ValueError):
+        PagedKVCache(8, 4, 4, 16, 8, 1, torch.float32, device="cpu", kv_rep=3)
+
+
+def test_install_sets_what_an_unedited_engine_cannot_say(monkeypatch):
+    for attr in ("default_kv_rep", "default_qk_normalised", "default_fuse_decode_append"):
+        monkeypatch.setattr(PagedKVCache, attr, getattr(PagedKVCache, attr))
+    for name in ("falcon_perception.kv_cache", "falcon_perception.paged_attention", "falcon_perception.attention"):
+        monkeypatch.delitem(sys.modules, name, raising=False)
+    bare = PagedKVCache(8, 4, 4, 16, 8, 1, torch.float32, device="cpu")
+    assert not bare.fuse_decode_append and not bare.qk_normalised and bare.score_bound(64, None) == 0.0
+    fpa.install(kv_rep=2, qk_norm=True)
+    c = PagedKVCache(8, 4, 4, 16, 64, 1, torch.float32, device="cpu")
+    assert c.fuse_decode_append and c.qk_normalised and c.kv_rep == 2
+    assert c.score_bound(64, None) == pytest.approx(1.1 * 8.0) and c.score_bound(64, 0.25) == pytest.approx(1.1 * 16.0)
+    fpa.install(fuse_decode_append=False)
+    c = PagedKVCache(8, 4, 4, 16, 64, 1, torch.float32, device="cpu")
+    assert not c.fuse_decode_append and not c.qk_normalised and c.kv_rep == 1
+
+
+def test_reserve_beyond_the_pool_raises_the_reference_message_on_a_dense_table():
+    """`paged_attention.py:138-143`: the message names the pages asked for and the pages left.  With the dense
+    table the pool always runs out before the table does; only a sparse table has a message of its own."""
+    c = PagedKVCache(8, 4, 4, 2, 8, 1, torch.float32, device="cpu")
+    b = c.allocate()
+    with pytest.raises(RuntimeError) as e:
+        c.reserve(b, None, 9 * 4)
+    assert str(e.value) == ("Cannot reserve 9 pages for a sequence of length 36 in batch 1. "
+                            "Only 7 pages available. Current capacity is 0 tokens.")
+    assert c.reserve(b, None, 9 * 4, dry_run=True) is False
+    sparse = PagedKVCache(64, 4, 4, 2, 8, 1, torch.float32, device="cpu", max_blocks_per_seq=3)
+    b = sparse.allocate()
+    with pytest.raises(RuntimeError, match="the page table holds 3 blocks"):
+        sparse.reserve(b, None, 16)
+    assert sparse.reserve(b, None, 16, dry_run=True) is False and sparse.reserve(b, None, 12, dry_run=True) is True
 
 
 def test_bench_reads_traffic_from_the_profiles_and_refuses_several_gpus():
