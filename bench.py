@@ -51,6 +51,10 @@ DECODE_WORKLOADS = {
     "cfg2f32": dict(seed=2, dtype="f32", B=64, Hq=16, Hc=8, D=128, P=128, n_pages=4096, prefix=1024, lo=64, hi=3072),
 }
 DTYPES = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
+# token ids of the synthetic packed rows (any five distinct values): start / end of an image block, a token
+# inside it, a text token, padding.  A span is [soi, eoi): the soi row is inside, the eoi row is not
+# (reference attention.py:77-79), and the text follows (data.py:513-522).
+SOI_ID, EOI_ID, IMG_ID, TXT_ID, PAD_ID = 3, 4, 7, 11, 0
 
 
 
@@ -264,6 +268,7 @@ class PrefillCase:
     # (the model's normalised q and k have sqrt(D) by construction; N(0, 1) rows are measured)
     score_bound: float = 0.0
     use_bound: bool = True
+    input_ids: torch.Tensor | None = None   # [1, Lq] int64 token ids the row limits follow from
 
     @property
     def page_size(self):
@@ -321,20 +326,23 @@ def make_prefill_case(name: str, device="cuda") -> PrefillCase:
     dgen = torch.Generator(device=device).manual_seed(c["seed"])
     cache.kv_cache.view(-1).normal_(generator=dgen)
     whole = c.get("whole", False)
-    bidx, pos, lim, pairs = [], [], [], 0
+    bidx, pos, lim, ids, pairs = [], [], [], [], 0
     for b, p in zip(slots, prefixes):
         if whole:  # all p + chunk rows in this step; rows of the image span [0, p) see the whole span
             n = p + chunk
             row_pos = list(range(n))
             row_lim = [max(t + 1, p) if t < p else t + 1 for t in range(n)]
+            row_ids = [SOI_ID] + [IMG_ID] * (p - 1) + [EOI_ID] + [TXT_ID] * (chunk - 1)
         else:      # only the chunk's rows; prefix already cached
             n = chunk
             row_pos = list(range(p, p + chunk))
             row_lim = [t + 1 for t in row_pos]
+            row_ids = [TXT_ID] * chunk
         gap = (-n) % 128
         bidx += [b] * n + [0] * gap
         pos += row_pos + [0] * gap
         lim += row_lim + [0] * gap
+        ids += row_ids + [PAD_ID] * gap
         pairs += sum(row_lim)
     Lq = len(bidx)
     q = torch.randn((1, c["Hq"], Lq, c["D"]), generator=dgen, device=device, dtype=torch.float32).to(dtype)
@@ -346,7 +354,7 @@ def make_prefill_case(name: str, device="cuda") -> PrefillCase:
                        torch.tensor([bidx], dtype=torch.int64, device=device),
                        torch.tensor([pos], dtype=torch.int64, device=device),
                        torch.tensor(lim, dtype=torch.int32, device=device), q, k_new, v_new, pairs,
-                       score_bound=bound)
+                       score_bound=bound, input_ids=torch.tensor([ids], dtype=torch.int64, device=device))
 
 
 # --------------------------------------------------------------------------
@@ -619,6 +627,96 @@ def prefill_rate(steps: int = 10, name: str = "cfg3") -> dict:
     return res
 
 
+def prefill_drop_in(steps: int = 5, name: str = "cfg3w", layers: int = MODEL_LAYERS) -> dict:
+    """A whole prefill step of the model's depth through the callables an unedited engine binds: one
+    `create_prefill_blockmask` from the token ids, then `insert_kv` + `compiled_flex_attn_prefill` for every layer
+    (reference paged_inference.py:637-733, model.py:150-162).  Wall clock with the host's part in it: Python,
+    ctypes, the row-limit kernel, the torch ops that turn packed limits into logical ones."""
+    from torch.nn.attention.flex_attention import AuxRequest
+
+    from falcon_perception_amd import attention as A
+    from falcon_perception_amd import ops
+    from falcon_perception_amd.paged_attention import PagedKVCache
+
+    one = make_prefill_case(name)
+    c = one.cfg
+    cache = PagedKVCache(one.cache.n_pages, c["P"], c["n_seq"] + 1, c["Hc"], c["D"], layers, DTYPES[c["dtype"]],
+                         device=one.q.device, qk_normalised=False)
+    cache.page_table.copy_(one.cache.page_table)
+    cache.page_table_cpu = [list(r) for r in one.cache.page_table_cpu]
+    cache.capacity = list(one.cache.capacity)
+    q, k_new, v_new, bidx, pos, ids = one.q, one.k_new, one.v_new, one.batch_idx, one.input_pos, one.input_ids
+    flops, bound, limits = one.flops(), one.score_bound, one.row_limit
+    del one
+    aux = AuxRequest(lse=True)
+    state = {}
+
+    def step():
+        mask = cache.create_prefill_blockmask(bidx, ids, SOI_ID, EOI_ID)
+        for layer in range(layers):
+            K, V = cache.insert_kv(layer, k_new, v_new, input_pos=pos, batch_idx=bidx)
+            A.compiled_flex_attn_prefill(q, K, V, block_mask=mask, return_aux=aux)
+        state["mask"] = mask
+
+    cache.score_bound = lambda head_dim, scale: bound  # what install(qk_norm=True) declares, for these N(0, 1) rows
+    step()
+    torch.cuda.synchronize()
+    real = bidx.view(-1) != 0  # padding rows (slot 0) are never looked at by the kernel
+    assert torch.equal(state["mask"].row_limit(pos, 0)[real], limits[real]), "the mask's row limits differ from the hand-written ones"
+    ms = time_steps(step, steps, 2, samples=7)
+    ms_mask = event_ms(lambda: cache.create_prefill_blockmask(bidx, ids, SOI_ID, EOI_ID), 20)
+    ms_limits = event_ms(lambda: ops.hybrid_row_limits(ids, SOI_ID, EOI_ID, bidx), 20, batch=4)
+    cache.check_prefill_masks()
+    res = {"workload": f"{name}: one prefill step of {layers} layers through create_prefill_blockmask, insert_kv and "
+                       "compiled_flex_attn_prefill (Python callables, eager, no host wait in the mask construction)",
+           "query_rows": int(q.shape[2]), "ms_per_step": ms, "ms_per_layer": ms / layers,
+           "tflops": layers * flops / (ms * 1e-3) / 1e12,
+           "frac_of_bf16_mfma_peak": layers * flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+           "create_prefill_blockmask_ms": ms_mask, "hybrid_row_limits_kernel_ms": ms_limits}
+    del cache
+    torch.cuda.empty_cache()
+    return res
+
+
+def decode_drop_in(case: "DecodeCase", steps: int) -> dict:
+    """The decode layer-step as an unedited engine runs it: `convert_logical_block_mask` once, then `insert_kv` +
+    `compiled_flex_attn_decode` (reference paged_inference.py:832-863, model.py:150-162), replayed from a captured
+    HIP graph; with the append left to the attention launch (what `install()` switches on) and launched on its own."""
+    from torch.nn.attention.flex_attention import AuxRequest, BlockMask
+
+    from falcon_perception_amd import attention as A
+
+    cache, B = case.cache, case.q.shape[0]
+    n_blocks = case.max_context // cache.page_size
+    full = cache.create_causal_blockmask(B=1, L=n_blocks * cache.page_size)
+    blk = (case.input_pos // cache.page_size).long()
+    zero = torch.zeros(B, dtype=torch.int64, device=case.q.device)
+    logical = BlockMask.from_kv_blocks(
+        full.kv_num_blocks[zero, :, blk].view(B, 1, 1), full.kv_indices[zero, :, blk].view(B, 1, 1, -1),
+        full.full_kv_num_blocks[zero, :, blk].view(B, 1, 1), full.full_kv_indices[zero, :, blk].view(B, 1, 1, -1),
+        BLOCK_SIZE=full.BLOCK_SIZE, mask_mod=lambda b, h, q, kv: q + case.input_pos[b] >= kv,
+        seq_lengths=(1, full.seq_lengths[1]))
+    aux = AuxRequest(lse=True)
+    pos = case.input_pos.view(B, 1)
+    saved = (cache.kv_rep, cache.fuse_decode_append)
+    cache.kv_rep = case.cfg.get("kv_rep", 1)
+
+    def step():
+        mask = cache.convert_logical_block_mask(logical, case.batch_idx)
+        K, V = cache.insert_kv(0, case.k_new, case.v_new, input_pos=pos, batch_idx=case.batch_idx)
+        return A.compiled_flex_attn_decode(case.q, K, V, block_mask=mask, return_aux=aux)
+
+    res = {}
+    for fused in (True, False):
+        cache.fuse_decode_append = fused
+        res["ms_hip_graph_append_in_attention" if fused else "ms_hip_graph_append_launch"] = graph_ms(step, steps)
+    cache.fuse_decode_append = True
+    res["ms_eager_append_in_attention"] = time_steps(step, steps, 10, samples=7)
+    cache.kv_rep, cache.fuse_decode_append = saved
+    cache.flush()
+    return res
+
+
 def small_batch_decode(steps: int = 200) -> dict:
     """The decode step (append + split-K pass + merge pass) of a few long sequences, replayed from a HIP
     graph: the regime of one or a few requests, where the split length and the merge pass set the time."""
@@ -631,6 +729,8 @@ def small_batch_decode(steps: int = 200) -> dict:
         ms = graph_ms(case.run_fused, steps)
         out[f"batch {B}, context ~{L}"] = {"split_tokens": case.split_tokens, "ms_per_step_hip_graph": ms,
                                           "gbps": case.bytes_decode() / (ms * 1e-3) / 1e9}
+        if (B, L) == (1, 8192):  # the same step through the callables an unedited engine binds
+            out[f"batch {B}, context ~{L}"]["drop_in"] = decode_drop_in(case, steps)
         del DECODE_WORKLOADS[name], case
         torch.cuda.empty_cache()
     return out
@@ -808,11 +908,88 @@ def cpu_baseline(case: DecodeCase, budget_s: float = 20.0, min_reps: int = 3) ->
     alg = (sum(ctx) * 2 * c["Hc"] * c["D"] * e + 2 * nb * c["Hq"] * c["D"] * e + 4 * nb * c["Hq"]
            + 8 * sum(math.ceil(x / c["P"]) for x in ctx) + 2 * nb * 2 * c["Hc"] * c["D"] * e + 8 * nb)
     return {
-        "value": alg / sec / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
+        "value": alg / sec / 1e9, "unit": "GB/s", "cores": cores, "cpu": cpu_model(), "kind": "port",
         "sample": f"{nb} of {c['B']} sequences of {case.name}, median of {reps} repetitions, one layer-step each "
                   f"(append + block-id gather + dense masked attention over the whole pool, fp32)",
         "decode_tok_s_per_layer": nb / sec, "ms_per_step_sample": sec * 1e3,
     }
+
+
+def cpu_model() -> str:
+    """Model name of the host processor, as /proc/cpuinfo states it."""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def summary_of(result: dict) -> dict:
+    """The figures of every leg in a few lines, as the LAST key of the output line: what is kept of a long line is
+    its end."""
+    def us(x):
+        return None if x is None else round(x * 1e3, 1)
+
+    def pct(x):
+        return None if x is None else round(100.0 * x, 1)
+
+    out = {"decode_step_us": {}, "decode_step_pct_of_hbm_peak": {}, "decode_kernel_pct_of_hbm_peak": {}}
+    wl = result["config"]["workload"].split(":")[0]
+    out["decode_step_us"][wl] = us(result["ms_per_step"])
+    out["decode_step_pct_of_hbm_peak"][wl] = round(result["pct_of_hbm_peak"], 1)
+    out["decode_kernel_pct_of_hbm_peak"][wl] = pct(result["roofline"]["frac"])
+    for name, leg in result.get("workloads", {}).items():
+        if "ms_per_step" in leg:
+            out["decode_step_us"][name] = us(leg["ms_per_step"])
+            out["decode_step_pct_of_hbm_peak"][name] = round(leg["pct_of_hbm_peak"], 1)
+            out["decode_kernel_pct_of_hbm_peak"][name] = pct(leg["roofline"]["frac"])
+    out["decode_step_variants_us"] = {
+        "separate_append_launch": us(result.get("ms_per_step_separate_append")),
+        "sink_gate_in_merge": us(result.get("ms_per_step_with_sink_gate")),
+        "hip_graph": us(result.get("ms_per_step_hip_graph")),
+        "all_layers_one_graph_per_layer": us(result["ms_all_layers_hip_graph"] / MODEL_LAYERS)
+        if result.get("ms_all_layers_hip_graph") else None}
+    if "decode_drop_in" in result:
+        out["decode_drop_in_us"] = {k: us(v) for k, v in result["decode_drop_in"].items()}
+    if "decode_small_batch" in result:
+        out["decode_small_batch_us"] = {}
+        for k, v in result["decode_small_batch"].items():
+            out["decode_small_batch_us"][k] = us(v["ms_per_step_hip_graph"])
+            if "drop_in" in v:
+                out["decode_small_batch_us"][k + " drop-in"] = {a: us(b) for a, b in v["drop_in"].items()}
+    out["tok_s"] = {"per_layer": round(result["decode_tok_s_per_layer"]), "model_measured": result.get("decode_tok_s_model_measured")}
+    pf = {}
+    for key in [k for k in result if k.startswith(("chunked_prefill", "prefill_whole_sequences"))]:
+        leg = result[key]
+        name = leg["workload"].split(":")[0]
+        frac = leg.get("frac_of_bf16_mfma_peak", leg.get("frac_of_f32_mfma_peak"))
+        pf[name] = {"us": us(leg["paged_prefill_ms"]), "tflops": round(leg["tflops"], 1), "pct_of_mfma_peak": pct(frac)}
+        if "paged_prefill_ms_no_score_bound" in leg:
+            pf[name]["us_no_score_bound"] = us(leg["paged_prefill_ms_no_score_bound"])
+    if pf:
+        out["prefill"] = pf
+    if "prefill_drop_in" in result:
+        d = result["prefill_drop_in"]
+        out["prefill_drop_in"] = {"us_per_layer": us(d["ms_per_layer"]), "pct_of_mfma_peak": pct(d["frac_of_bf16_mfma_peak"]),
+                                  "create_prefill_blockmask_us": us(d["create_prefill_blockmask_ms"]),
+                                  "hybrid_row_limits_kernel_us": us(d["hybrid_row_limits_kernel_ms"])}
+    if "cfg4_mixed_step" in result:
+        out["cfg4_mixed_step_us"] = us(result["cfg4_mixed_step"].get("ms_per_mixed_step"))
+    ps = result.get("prefill_sized", {})
+    if ps:
+        out["pieces_pct_of_hbm_peak"] = {k[:-len("_frac_of_peak")]: pct(v) for k, v in ps.items() if k.endswith("_frac_of_peak")}
+    cb = {}
+    if "cpu_baseline" in result:
+        cb[wl] = {k: result["cpu_baseline"][k] for k in ("value", "unit", "cores", "cpu")}
+    for name, leg in result.get("workloads", {}).items():
+        if "cpu_baseline" in leg:
+            cb[name] = {k: leg["cpu_baseline"][k] for k in ("value", "unit", "cores")}
+    if cb:
+        out["cpu_baseline"] = cb
+    return out
 
 
 def calibration_copies() -> None:
@@ -919,6 +1096,7 @@ def main() -> int:
         result["cpu_baseline"] = cpu_baseline(case)
         result["gpu_over_cpu"] = value / result["cpu_baseline"]["value"]
     if not args.decode_only:
+        result["decode_drop_in"] = decode_drop_in(case, args.steps)
         ms_model = model_depth_graph_ms(case, args.steps)  # takes and returns 56 GiB
         if ms_model is not None:
             result["ms_all_layers_hip_graph"] = ms_model
@@ -943,6 +1121,8 @@ def main() -> int:
         result["prefill_whole_sequences_expanded_heads"] = prefill_rate(name="cfg3wx")
         result["prefill_whole_sequences_head_dim_64"] = prefill_rate(name="cfg3wd64")
         result["decode_small_batch"] = small_batch_decode()
+        result["prefill_drop_in"] = prefill_drop_in()
+    result["summary"] = summary_of(result)
     print(json.dumps(result))
     return 0
 

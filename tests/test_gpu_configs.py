@@ -156,3 +156,62 @@ def test_cfg5_long_context_decode_on_a_pool_sized_to_hbm():
                               case.page_size, case.max_context, split_tokens=512)
     np.testing.assert_allclose(l2.cpu().numpy(), lse.cpu().numpy(), atol=1e-4, rtol=1e-5)
     np.testing.assert_allclose(f64(o2), f64(out), atol=8e-3, rtol=8e-3)
+
+
+@pytest.mark.parametrize("name", ["cfg3w", "cfg3wx", "cfg3wd64"])
+@pytest.mark.parametrize("bounded", [False, True], ids=["running-maximum", "score-bound"])
+def test_whole_sequence_prefill_at_full_size(name, bounded):
+    """The prefill step the reference's engine runs (whole sequences packed, each padded to 128,
+    paged_inference.py:637-672) at the size the bench times: 8 sequences of an image span of U[256, 4096] tokens
+    plus 512 text tokens, 23040 packed rows, 16 query heads; on 8 cached heads, on the engine's 16, at head_dim 64.
+    Everything goes through the drop-in: the mask from the token ids (`create_prefill_blockmask` -> row-limit
+    kernel -> `row_limit`), `insert_kv`, `compiled_flex_attn_prefill`.  Checked: the limits against the oracle's
+    (and against the ones the bench writes by hand), the pool against the rows, and sampled rows of three
+    sequences -- inside the span (first, middle, last), the end-of-image row, the first and the last text row --
+    against the float64 oracle."""
+    import bench
+    from torch.nn.attention.flex_attention import AuxRequest
+
+    from falcon_perception_amd import attention as A
+    from tests.test_gpu_prefill import BOUNDED_LSE_ATOL
+
+    case = bench.make_prefill_case(name, device=DEV)
+    cache = case.cache
+    bidx = case.batch_idx.cpu().numpy().reshape(-1)
+    ids = case.input_ids.cpu().numpy().reshape(-1)
+    pos = case.input_pos.cpu().numpy().reshape(-1)
+    L = len(ids)
+    assert L == 23040 and case.q.shape[2] == L
+
+    mask = cache.create_prefill_blockmask(case.batch_idx, case.input_ids, bench.SOI_ID, bench.EOI_ID)
+    hi, status = O.chunk_row_limits(bidx, ids, bench.SOI_ID, bench.EOI_ID)
+    assert status == 0
+    assert np.array_equal(mask.row_hi.cpu().numpy(), hi)
+    limits = (pos + hi - np.arange(L)).astype(np.int32)  # logical: position + reach beyond the row
+    assert np.array_equal(mask.row_limit(case.input_pos, 0).cpu().numpy(), limits)
+    real = bidx != 0
+    assert np.array_equal(case.row_limit.cpu().numpy()[real], limits[real])
+
+    if bounded:
+        cache.score_bound = lambda head_dim, scale: case.score_bound  # a bound that holds for these N(0, 1) rows
+    K, V = cache.insert_kv(0, case.k_new, case.v_new, input_pos=case.input_pos, batch_idx=case.batch_idx)
+    out, aux = A.compiled_flex_attn_prefill(case.q, K, V, block_mask=mask, return_aux=AuxRequest(lse=True))
+    cache.check_prefill_masks()
+
+    pk, pv = case.pool_k.float().cpu().numpy(), case.pool_v.float().cpu().numpy()
+    pt = case.page_table.cpu().numpy()
+    rows = []
+    for s in (0, 3, len(case.slots) - 1):
+        r = np.flatnonzero(bidx == case.slots[s])
+        p = case.prefixes[s]
+        rows += [r[0], r[p // 2], r[p - 1], r[p], r[p + 1], r[-1]]
+        # the rows just appended are the keys the attention read
+        slots_of = pt[case.slots[s], pos[r] // case.page_size] * case.page_size + pos[r] % case.page_size
+        assert np.array_equal(pk[:, slots_of], case.k_new[0][:, r].float().cpu().numpy())
+    rows = np.array(sorted(rows))
+    eo, el = O.prefill_attention_paged(f64(case.q[:, :, rows]), pk, pv, pt, bidx[rows], None, limits[rows], case.page_size)
+    go, gl = f64(out[:, :, rows]), f64(aux.lse[:, :, rows])
+    np.testing.assert_allclose(go, eo, atol=ATOL, rtol=RTOL)
+    np.testing.assert_allclose(gl, el, atol=BOUNDED_LSE_ATOL if bounded else 2e-3, rtol=RTOL)
+    pad = np.flatnonzero(~real)
+    assert not f64(out[:, :, pad]).any() and np.isneginf(f64(aux.lse[:, :, pad])).all()
