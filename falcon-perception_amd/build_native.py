@@ -10,6 +10,7 @@ from __future__ import annotations
 
 import concurrent.futures
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -30,6 +31,9 @@ FLAGS = [
     "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    # one remark per kernel with its registers, LDS and scratch: kept beside the object file
+    # (build/<source>.resources.txt) and read back by `resource_usage()`
+    "-Rpass-analysis=kernel-resource-usage",
     "-I", INCLUDE,
     "-I", CSRC,
 ]
@@ -52,7 +56,28 @@ def _compile(src: str) -> str:
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{res.stdout}\n{res.stderr}")
+    with open(obj[:-2] + ".resources.txt", "w") as f:
+        f.write(res.stderr)
     return obj
+
+
+def resource_usage() -> dict[str, dict[str, int]]:
+    """Per kernel of the last build: {"vgprs", "agprs", "scratch" (bytes per lane), "lds" (bytes per workgroup),
+    "occupancy" (wavefronts per SIMD)}, keyed by the mangled kernel name; builds first if nothing has been
+    built.  A kernel with scratch > 0 spills registers to memory; the first launch of such a kernel makes the
+    runtime set that memory up, which it cannot do while a stream is being captured into a graph."""
+    names = [os.path.join(OBJ_DIR, os.path.basename(s)[:-4] + ".resources.txt") for s in sources()]
+    if not all(os.path.exists(n) for n in names):
+        build_library(verbose=False)
+    out: dict[str, dict[str, int]] = {}
+    fields = {"vgprs": r"VGPRs: (\d+)", "agprs": r"AGPRs: (\d+)", "scratch": r"ScratchSize \[bytes/lane\]: (\d+)",
+              "lds": r"LDS Size \[bytes/block\]: (\d+)", "occupancy": r"Occupancy \[waves/SIMD\]: (\d+)"}
+    for n in names:
+        with open(n) as f:
+            text = f.read()
+        for block in re.split(r"remark: [^\n]*Function Name: ", text)[1:]:
+            out[block.split()[0]] = {k: int(re.search(v, block).group(1)) for k, v in fields.items()}
+    return out
 
 
 def build_library(verbose: bool = True) -> str:

@@ -10,8 +10,17 @@
  * Conventions
  *  - Every pointer is a DEVICE pointer owned by the caller.  The library
  *    borrows it for the duration of the launch; it allocates and frees nothing.
- *  - `stream` is a hipStream_t passed as void*.  All work is enqueued on it,
- *    nothing synchronises, so every entry point may be captured in a HIP graph.
+ *  - `stream` is a hipStream_t passed as void*.  All work is enqueued on it and
+ *    nothing synchronises, so the entry points may be captured in a HIP graph.  One
+ *    condition: a kernel that keeps spilled registers in scratch memory must have been
+ *    launched once on the device BEFORE a capture, because its first launch makes the
+ *    runtime set that memory up, which it cannot do while a stream is being captured.
+ *    The only such kernels here are those fp_paged_prefill launches at head_dim 64 for a
+ *    launch that is not cut along the keys (bf16 and f16, 20 to 36 bytes per lane); every
+ *    kernel behind the other entry points, and the rest of fp_paged_prefill, uses none
+ *    (the build writes every kernel's figure to build/<source>.resources.txt and a test
+ *    holds the list to exactly this).  The reference's engine captures decode steps only
+ *    (paged_inference.py:916-935).
  *  - Strides are in ELEMENTS of the tensor's dtype, the innermost (head_dim)
  *    stride must be 1.
  *  - Return value: 0 on success, a negative FP_ERR_* code otherwise;
@@ -260,7 +269,9 @@ int fp_paged_decode_append(const void* k_new, const void* v_new,
  * in the reference.  The split-K partial results go to an array of FP_NOALLOC_SCRATCH_BYTES that is
  * part of the library's device image (every GPU the library runs on holds its own copy until the
  * process ends); the call allocates and frees nothing.  The first call on a device looks the array's
- * address up once (hipGetSymbolAddress, with that device current).
+ * address up once (hipGetSymbolAddress, with that device current), which may make the runtime load the
+ * library's device image: make that first call OUTSIDE a graph capture (any small launch will do);
+ * every later call on the device may be captured.
  *  - A launch whose partial results (fp_paged_decode_workspace_bytes for the same shape) exceed
  *    FP_NOALLOC_SCRATCH_BYTES is refused with FP_ERR_WORKSPACE.
  *  - All calls on one GPU share that GPU's array: calls that overlap there (different streams or

@@ -13,6 +13,8 @@ for p in (ROOT, os.path.join(ROOT, "falcon-perception_amd")):
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+    config.addinivalue_line("markers", "bigmem: holds tens of GB of HBM and asserts that they are free: needs a GPU "
+                                       "no other process is using (deselect with -m 'gpu and not bigmem')")
 
 
 def pytest_collection_modifyitems(config, items):

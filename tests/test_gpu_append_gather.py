@@ -222,6 +222,7 @@ def test_large_append_round_trip_and_checksum():
     assert int(pv.view(torch.int16).to(torch.int64).sum()) == int(v.view(torch.int16).to(torch.int64).sum())
 
 
+@pytest.mark.bigmem
 def test_append_and_gather_with_more_than_2_32_vectors_in_a_launch():
     """Rows of 3 bf16 values move as 2-byte vectors, one per lane; 1 435 000 000 such rows are more than
     2^32 lanes in one launch, the case in which the kernels index their lanes with 64 bits.  One sequence

@@ -130,6 +130,7 @@ def test_cfg4_continuous_batching_churn():
         assert len(live) + cache.num_free_pages == n_pages - 1
 
 
+@pytest.mark.bigmem
 def test_cfg5_long_context_decode_on_a_pool_sized_to_hbm():
     import bench
 

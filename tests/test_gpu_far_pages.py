@@ -49,6 +49,7 @@ def same_pool(small, large):
     assert not large[:, :lo].view(torch.int16).any()
 
 
+@pytest.mark.bigmem
 def test_every_kernel_on_pages_beyond_4_gib():
     free, _ = torch.cuda.mem_get_info()
     assert free > 60e9, f"only {free / 1e9:.0f} GB of HBM free: this case holds about 30 GB"

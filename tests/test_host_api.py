@@ -400,3 +400,29 @@ def test_hybrid_row_limits_argument_errors(native_lib):
     assert native_lib.fp_hybrid_row_limits(None, None, None, 0, 70000, 1, 2, None, None, None) == -2
     assert native_lib.fp_hybrid_row_limits(None, None, None, 0, 0, 1, 2, None, None, None) == 0  # an empty row is fine
     assert native_lib.fp_hybrid_row_limits(None, None, None, 0, 5, 1, 2, None, None, None) == -1  # null pointers
+
+
+def test_only_the_documented_kernels_use_scratch_memory():
+    """A kernel whose registers spill to scratch memory cannot be launched for the first time while a stream
+    is being captured into a graph (the runtime sets the memory up at that launch).  The header promises that
+    this concerns nothing but the four-wavefront instances of the 16-bit prefill kernel at head_dim 64; the
+    compiler's own report of every kernel of the last build is held against that promise."""
+    import importlib.util
+    import re
+
+    spec = importlib.util.spec_from_file_location("fp_build_native", os.path.join(ROOT, "falcon-perception_amd", "build_native.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    usage = mod.resource_usage()
+    assert len(usage) > 300  # every template instance of the eight sources
+    for family in ("paged_decode_kernel", "paged_decode_merge", "kv_append_kernel", "kv_gather_kernel", "qkv_rope",
+                   "hybrid_row_limits_kernel", "convert_block_ids_kernel", "paged_prefill_kernel", "paged_prefill_f32_kernel",
+                   "paged_prefill_merge_kernel"):
+        assert any(family in name for name in usage), family
+    # paged_prefill_kernel<E, 64, G, pow2, 4 wavefronts, bounded>
+    allowed = re.compile(r"paged_prefill_kernelINS_\d?(BF16|F16)ELi64ELi\dELb[01]ELi4ELb[01]E")
+    spilling = {name: u["scratch"] for name, u in usage.items() if u["scratch"] > 0}
+    assert spilling, "the header's exception list can go: no kernel uses scratch any more"
+    for name, scratch in spilling.items():
+        assert allowed.search(name), f"{name} spills {scratch} bytes per lane and may be launched under graph capture"
+        assert scratch <= 64

@@ -68,3 +68,27 @@ def test_a_launch_beyond_the_array_is_refused():
     table = torch.zeros((4, 8192 // 16), dtype=torch.int64, device=DEV)
     with pytest.raises(RuntimeError, match="the library's array holds"):
         ops.paged_decode_noalloc(qq, pool, pool, table, bb, pp, 16, ctx, out, lse, split_tokens=split)
+
+
+def test_captured_in_a_graph_after_a_first_call_outside():
+    """The first call on a device resolves the array's address and belongs outside a capture; after it the
+    entry point is captured like any other: three replays with other positions and queries in between, each
+    bit-identical to fp_paged_decode run eagerly on the same inputs."""
+    st, q, pos, bidx = case(56, 9, 700, 4, 2, 128, 32, torch.bfloat16)
+    pk, pv = st.pool_planes()
+    lens = pos + 1
+    out = torch.empty_like(q)
+    lse = torch.empty((q.shape[0], q.shape[1], 1), dtype=torch.float32, device=DEV)
+    run = lambda: ops.paged_decode_noalloc(q, pk, pv, st.cache.page_table, bidx, pos, st.P, 704, out, lse, split_tokens=128)
+    run()  # outside the capture
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        run()
+    for i in range(3):
+        pos.copy_(torch.clamp(lens - 1 - 37 * i, min=0))
+        q.copy_(randn(st.gen, tuple(q.shape), torch.bfloat16).to(DEV))
+        g.replay()
+        torch.cuda.synchronize()
+        ref_out, ref_lse = ops.paged_decode(q, pk, pv, st.cache.page_table, bidx, pos, st.P, 704, split_tokens=128)
+        assert torch.equal(out, ref_out) and torch.equal(lse, ref_lse), i
