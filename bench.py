@@ -584,9 +584,11 @@ def append_gather_rates(steps: int = 20, T: int = 32768, H: int = 16, D: int = 1
             "kv_gather_cold_frac_of_peak": bytes_g / (ms_g_cold * 1e-3) / 1e9 / HBM_PEAK_GBPS}
 
 
-def prefill_rate(steps: int = 10, name: str = "cfg3") -> dict:
-    """Chunked prefill at BASELINE configs[2]: append the 512-token chunks, attend over the paged prefix."""
+def prefill_rate(steps: int = 10, name: str = "cfg3", bounded: bool = True, both: bool = True) -> dict:
+    """Chunked prefill at BASELINE configs[2]: append the 512-token chunks, attend over the paged prefix.
+    `bounded`: declare the score bound (bf16); `both`: time the other variant beside it."""
     case = make_prefill_case(name)
+    case.use_bound = bounded
     case.append()
     for _ in range(3):
         case.attend()
@@ -594,7 +596,7 @@ def prefill_rate(steps: int = 10, name: str = "cfg3") -> dict:
     ms_a = event_ms(case.append, steps)
     tf = case.flops() / (ms * 1e-3) / 1e12
     ms_unbounded = None
-    if case.q.dtype == torch.bfloat16:  # the same launch without the score bound: online softmax with a running maximum
+    if case.q.dtype == torch.bfloat16 and bounded and both:  # the same launch without the score bound: online softmax with a running maximum
         ms_unbounded = event_ms(lambda: case.attend(bounded=False), steps, batch=4)
     what = {"cfg3": "cfg3: 8 sequences, paged prefix U[256,4096], 512-token chunk each, 16 q / 8 kv heads, D 128",
             "cfg3w": "cfg3w: the same 8 sequences prefilled whole (prefix + chunk rows in one step, prefix rows see "
@@ -727,8 +729,12 @@ def small_batch_decode(steps: int = 200) -> dict:
                                       n_pages=B * (L // 128 + 2) + 8, prefix=L - 64, lo=0, hi=63)
         case = make_decode_case(name)
         ms = graph_ms(case.run_fused, steps)
+        # one step per replay pays the replay's own launch cost (about 5 us) on a 12 us step; the engine replays a
+        # graph of the model's depth, so the same step is also timed as one of 28 layers (own K/V planes each)
+        ms_model = model_depth_graph_ms(case, steps)
         out[f"batch {B}, context ~{L}"] = {"split_tokens": case.split_tokens, "ms_per_step_hip_graph": ms,
-                                          "gbps": case.bytes_decode() / (ms * 1e-3) / 1e9}
+                                          "gbps": case.bytes_decode() / (ms * 1e-3) / 1e9,
+                                          "ms_per_layer_in_a_graph_of_all_layers": ms_model / MODEL_LAYERS if ms_model else None}
         if (B, L) == (1, 8192):  # the same step through the callables an unedited engine binds
             out[f"batch {B}, context ~{L}"]["drop_in"] = decode_drop_in(case, steps)
         del DECODE_WORKLOADS[name], case
@@ -958,6 +964,7 @@ def summary_of(result: dict) -> dict:
         out["decode_small_batch_us"] = {}
         for k, v in result["decode_small_batch"].items():
             out["decode_small_batch_us"][k] = us(v["ms_per_step_hip_graph"])
+            out["decode_small_batch_us"][k + ", per layer in a graph of all layers"] = us(v.get("ms_per_layer_in_a_graph_of_all_layers"))
             if "drop_in" in v:
                 out["decode_small_batch_us"][k + " drop-in"] = {a: us(b) for a, b in v["drop_in"].items()}
     out["tok_s"] = {"per_layer": round(result["decode_tok_s_per_layer"]), "model_measured": result.get("decode_tok_s_model_measured")}
@@ -1018,6 +1025,8 @@ def main() -> int:
     ap.add_argument("--hbm-budget-gb", type=float, default=None, help="pool size for cfg5 (default: what fits, at most 180)")
     ap.add_argument("--prefill-only", default=None, choices=sorted(PREFILL_WORKLOADS),
                     help="time only the chunked-prefill attention of this workload and print its JSON (for profiling)")
+    ap.add_argument("--no-score-bound", action="store_true",
+                    help="with --prefill-only: leave the score bound out (the online softmax with a running maximum)")
     ap.add_argument("--pieces-only", action="store_true",
                     help="time only KV append, page gather and the fused norm + rotary append at 32768 tokens and print "
                          "their JSON (for profiling)")
@@ -1037,7 +1046,7 @@ def main() -> int:
     if args.pmc_calibration:
         calibration_copies()
     if args.prefill_only:
-        print(json.dumps(prefill_rate(max(args.steps, 1), args.prefill_only)))
+        print(json.dumps(prefill_rate(max(args.steps, 1), args.prefill_only, bounded=not args.no_score_bound, both=False)))
         return 0
     if args.pieces_only:
         print(json.dumps(append_gather_rates(max(args.steps, 1))))
