@@ -834,11 +834,18 @@ def cfg4_mixed_step(steps: int = 6) -> dict:
         out4 = torch.empty_like(q4)
         lse4 = torch.empty((1, Hq, 4096), dtype=torch.float32, device=dev)
 
+        # a bound of |scale * q.k| that holds for the rows of this step (N(0, 1) everywhere, stale pages included)
+        if step == 0:
+            k_norm = float(pk.float().norm(dim=-1).max())
+        k_norm = max(k_norm, float(k4.float().norm(dim=-1).max()), float(k1.float().norm(dim=-1).max()))
+        bound = float(q4.float().norm(dim=-1).max()) * k_norm / math.sqrt(D)
+
         def mixed():
             ops.paged_decode(q1, pk, pv, cache.page_table, bt, pt, P, max_context, split_tokens=split, workspace=ws,
                              out=out1, lse=lse1, k_new=k1, v_new=v1)
             cache.insert_kv(0, k4, v4, input_pos=pos, batch_idx=bidx)
-            ops.paged_prefill(q4, pk, pv, cache.page_table, bidx, lim, P, out=out4, lse=lse4, workspace=pws)
+            ops.paged_prefill(q4, pk, pv, cache.page_table, bidx, lim, P, out=out4, lse=lse4, workspace=pws,
+                              score_bound=bound)
 
         if step == 0:
             warm_clocks(mixed)
@@ -919,6 +926,85 @@ def cpu_baseline(case: DecodeCase, budget_s: float = 20.0, min_reps: int = 3) ->
                   f"(append + block-id gather + dense masked attention over the whole pool, fp32)",
         "decode_tok_s_per_layer": nb / sec, "ms_per_step_sample": sec * 1e3,
     }
+
+
+def row_limits_rate(L: int, steps: int = 50) -> dict:
+    """The row-limit kernel behind `create_prefill_blockmask` alone, on a packed row of L tokens: sequences of
+    4096 tokens, each an image block of 3000 tokens and text, with their cache slots."""
+    from falcon_perception_amd import ops
+
+    ids = torch.full((L,), TXT_ID, dtype=torch.int64, device="cuda")
+    bidx = torch.ones(L, dtype=torch.int64, device="cuda")
+    for s0 in range(0, L, 4096):
+        ids[s0] = SOI_ID
+        ids[s0 + 1:s0 + 3000] = IMG_ID
+        ids[min(s0 + 3000, L - 1)] = EOI_ID
+        bidx[s0:s0 + 4096] = 1 + s0 // 4096
+    status = torch.zeros(1, dtype=torch.int32, device="cuda")
+    ms = event_ms(lambda: ops.hybrid_row_limits(ids, SOI_ID, EOI_ID, bidx, None, status), steps, batch=4)
+    return {"kernel": "hybrid_row_limits_kernel", "rows": L, "ms": ms, "status": int(status.item())}
+
+
+def shader_clock_mhz() -> float | None:
+    """Current shader clock of GPU 0 as the driver reports it (the starred level of pp_dpm_sclk), or None."""
+    import glob
+
+    for path in sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk")):
+        try:
+            with open(path) as f:
+                for line in f:
+                    if line.rstrip().endswith("*"):
+                        return float(line.split(":")[1].strip().split("M")[0])
+        except (OSError, ValueError, IndexError):
+            continue
+    return None
+
+
+def clock_probe(seconds: float = 2.0) -> dict:
+    """Launches of identical prefill workgroups -- n sequences of a 512-row chunk over a 4096-token prefix, 32
+    workgroups each, not cut along the keys -- back to back for `seconds` per size, with the shader clock read
+    from the driver every 50 ms meanwhile: what a launch of the same workgroups costs as more of the chip is busy."""
+    import threading
+
+    from falcon_perception_amd import ops
+
+    out = {}
+    for n_seq in (1, 2, 4, 6, 8, 16):
+        name = f"probe_{n_seq}"
+        PREFILL_WORKLOADS[name] = dict(seed=3, dtype="bf16", n_seq=n_seq, Hq=16, Hc=8, D=128, P=128, prefix_lo=4096,
+                                       prefix_hi=4096, chunk=512)
+        case = make_prefill_case(name)
+        case.append()
+        run = lambda: ops.paged_prefill(case.q, case.pool_k, case.pool_v, case.cache.page_table, case.batch_idx,
+                                        case.row_limit, case.page_size, workspace=False, score_bound=case.score_bound)
+        clocks, stop = [], threading.Event()
+
+        def sample():
+            while not stop.is_set():
+                mhz = shader_clock_mhz()
+                if mhz is not None:
+                    clocks.append(mhz)
+                time.sleep(0.05)
+
+        warm_clocks(run)
+        th = threading.Thread(target=sample)
+        th.start()
+        n, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(50):
+                run()
+            torch.cuda.synchronize()
+            n += 50
+        dt = time.perf_counter() - t0
+        stop.set()
+        th.join()
+        out[f"{32 * n_seq} workgroups"] = {
+            "us_per_launch": dt / n * 1e6, "tflops": case.flops() / (dt / n) / 1e12,
+            "sclk_mhz_median": statistics.median(clocks) if clocks else None,
+            "sclk_mhz_min": min(clocks) if clocks else None, "sclk_samples": len(clocks)}
+        del PREFILL_WORKLOADS[name], case
+        torch.cuda.empty_cache()
+    return out
 
 
 def cpu_model() -> str:
@@ -1027,6 +1113,11 @@ def main() -> int:
                     help="time only the chunked-prefill attention of this workload and print its JSON (for profiling)")
     ap.add_argument("--no-score-bound", action="store_true",
                     help="with --prefill-only: leave the score bound out (the online softmax with a running maximum)")
+    ap.add_argument("--row-limits-only", type=int, default=None, metavar="ROWS",
+                    help="time only the row-limit kernel of create_prefill_blockmask on a packed row of ROWS tokens")
+    ap.add_argument("--clock-probe", action="store_true",
+                    help="launches of identical prefill workgroups at 32 .. 512 workgroups with the shader clock sampled "
+                         "from the driver meanwhile, as JSON")
     ap.add_argument("--pieces-only", action="store_true",
                     help="time only KV append, page gather and the fused norm + rotary append at 32768 tokens and print "
                          "their JSON (for profiling)")
@@ -1050,6 +1141,12 @@ def main() -> int:
         return 0
     if args.pieces_only:
         print(json.dumps(append_gather_rates(max(args.steps, 1))))
+        return 0
+    if args.row_limits_only:
+        print(json.dumps(row_limits_rate(args.row_limits_only, max(args.steps, 1))))
+        return 0
+    if args.clock_probe:
+        print(json.dumps(clock_probe()))
         return 0
     case = make_decode_case(args.workload, hbm_budget_gb=args.hbm_budget_gb)
     c = case.cfg
