@@ -606,42 +606,73 @@ __global__ __launch_bounds__(kThreads, (decode_waves_per_simd<E, D, G, kPerHeadK
 }
 
 // ---- cross-split merge ------------------------------------------------------
+// One batch of kBatch consecutive splits of a partial row, as this lane holds it.
+template <int D, int kBatch>
+struct SplitBatch {
+  float m[kBatch], l[kBatch], acc[kBatch][(D + 63) / 64];
+};
+
+// Requests the splits base .. base + kBatch - 1 (those below `limit`) of partial row p0.
+template <int D, int kBatch>
+__device__ __forceinline__ void load_batch(const DecodeArgs& a, int64_t p0, int base, int limit, int64_t row_stride,
+                                           SplitBatch<D, kBatch>& t) {
+  constexpr int DPL = (D + 63) / 64;
+#pragma unroll
+  for (int s = 0; s < kBatch; ++s) {
+    const bool on = base + s < limit;
+    const int64_t p = p0 + (on ? base + s : 0) * row_stride;
+    t.m[s] = on ? a.ws_ml[p * 2] : -INFINITY;
+    t.l[s] = on ? a.ws_ml[p * 2 + 1] : 0.f;
+#pragma unroll
+    for (int j = 0; j < DPL; ++j) {
+      const int d = (threadIdx.x & 63) + j * 64;
+      t.acc[s][j] = (on && d < D) ? a.ws_acc[p * D + d] : 0.f;
+    }
+  }
+}
+
+// Folds the splits of a batch that lie below ns into the running state (m_run, den, num) of this lane.  A batch
+// that was requested before ns was known may hold rows of splits the sequence does not have (whatever the
+// workspace held): they are dropped here by selects and never enter the arithmetic.
+template <int D, int kBatch>
+__device__ __forceinline__ void fold_batch(SplitBatch<D, kBatch>& t, int base, int ns, float& m_run, float& den,
+                                           float (&num)[(D + 63) / 64]) {
+  constexpr int DPL = (D + 63) / 64;
+  float mn = m_run;
+#pragma unroll
+  for (int s = 0; s < kBatch; ++s) {
+    if (base + s >= ns) {
+      t.m[s] = -INFINITY;
+      t.l[s] = 0.f;
+#pragma unroll
+      for (int j = 0; j < DPL; ++j) t.acc[s][j] = 0.f;
+    }
+    mn = fmaxf(mn, t.m[s]);
+  }
+  const float ms = safe_max(mn);
+  const float keep = fast_exp2(m_run - ms);  // 0 while the state is empty
+  den *= keep;
+#pragma unroll
+  for (int j = 0; j < DPL; ++j) num[j] *= keep;
+#pragma unroll
+  for (int s = 0; s < kBatch; ++s) {
+    const float wgt = fast_exp2(t.m[s] - ms);
+    den += t.l[s] * wgt;
+#pragma unroll
+    for (int j = 0; j < DPL; ++j) num[j] += t.acc[s][j] * wgt;
+  }
+  m_run = mn;
+}
+
 // Folds the splits first, first + stride, ... (kBatch consecutive splits each time, below ns) of partial
 // row p0 into the running state (m_run, den, num) of this lane; scores are in log2 units.
 template <int D, int kBatch>
 __device__ __forceinline__ void merge_batches(const DecodeArgs& a, int64_t p0, int first, int stride, int ns, float& m_run,
                                               float& den, float (&num)[(D + 63) / 64], int64_t row_stride = 1) {
-  constexpr int DPL = (D + 63) / 64;
   for (int base = first; base < ns; base += stride) {
-    float m_s[kBatch], l_s[kBatch], acc_s[kBatch][DPL];
-#pragma unroll
-    for (int s = 0; s < kBatch; ++s) {
-      const bool on = base + s < ns;
-      const int64_t p = p0 + (on ? base + s : 0) * row_stride;
-      m_s[s] = on ? a.ws_ml[p * 2] : -INFINITY;
-      l_s[s] = on ? a.ws_ml[p * 2 + 1] : 0.f;
-#pragma unroll
-      for (int j = 0; j < DPL; ++j) {
-        const int d = (threadIdx.x & 63) + j * 64;
-        acc_s[s][j] = (on && d < D) ? a.ws_acc[p * D + d] : 0.f;
-      }
-    }
-    float mn = m_run;
-#pragma unroll
-    for (int s = 0; s < kBatch; ++s) mn = fmaxf(mn, m_s[s]);
-    const float ms = safe_max(mn);
-    const float keep = fast_exp2(m_run - ms);  // 0 while the state is empty
-    den *= keep;
-#pragma unroll
-    for (int j = 0; j < DPL; ++j) num[j] *= keep;
-#pragma unroll
-    for (int s = 0; s < kBatch; ++s) {
-      const float wgt = fast_exp2(m_s[s] - ms);
-      den += l_s[s] * wgt;
-#pragma unroll
-      for (int j = 0; j < DPL; ++j) num[j] += acc_s[s][j] * wgt;
-    }
-    m_run = mn;
+    SplitBatch<D, kBatch> t;
+    load_batch<D, kBatch>(a, p0, base, ns, row_stride, t);
+    fold_batch<D, kBatch>(t, base, ns, m_run, den, num);
   }
 }
 
@@ -666,73 +697,27 @@ __global__ __launch_bounds__(64) void paged_decode_merge_kernel(const DecodeArgs
   const int b = blockIdx.y;
   const int64_t p0 = (static_cast<int64_t>(b) * a.Hq + hq) * a.n_splits;
 
-  // The kernel is a chain of memory latencies, so when the launch has at most kBatch splits every
-  // load is requested at once, the partials of splits this sequence does not have included (they are
-  // dropped by a select once its length is known, never used in arithmetic).
+  // The kernel is a chain of memory latencies, so the first kBatch splits are requested together with the
+  // sequence's position, by the launch's split count: the partials of splits this sequence does not have
+  // are dropped by selects once its length is known and never enter the arithmetic.
   constexpr int kBatch = 8;
   constexpr int DPL = (D + 63) / 64;  // output elements per lane
-  const bool batched = a.n_splits <= kBatch;
-  float m_s[kBatch], l_s[kBatch], acc_s[kBatch][DPL];
-  if (batched) {
-#pragma unroll
-    for (int s = 0; s < kBatch; ++s) {
-      const bool on = s < a.n_splits;
-      m_s[s] = on ? a.ws_ml[(p0 + s) * 2] : -INFINITY;
-      l_s[s] = on ? a.ws_ml[(p0 + s) * 2 + 1] : 0.f;
-#pragma unroll
-      for (int j = 0; j < DPL; ++j) {
-        const int d = threadIdx.x + j * 64;
-        acc_s[s][j] = (on && d < D) ? a.ws_acc[(p0 + s) * D + d] : 0.f;
-      }
-    }
-  }
-
   int64_t L = fp::load_index(a.input_pos, b, a.pos_i64) + 1;
   const int64_t trow = a.batch_idx[b];
+  SplitBatch<D, kBatch> first;
+  load_batch<D, kBatch>(a, p0, 0, a.n_splits, 1, first);
   if (trow < 0 || trow >= a.max_batch) L = 0;
   if (L > a.max_context) L = a.max_context;
   const int part = split_part(static_cast<int>(L), a.split_tokens);
   const int ns = L <= 0 ? 0 : static_cast<int>((L + part - 1) / part);
 
-  if (batched) {
-    float mn = -INFINITY;
-#pragma unroll
-    for (int s = 0; s < kBatch; ++s) {
-      if (s >= ns) m_s[s] = -INFINITY;
-      mn = fmaxf(mn, m_s[s]);
-    }
-    const float ms = safe_max(mn);
-    float den = 0.f, num[DPL];
-#pragma unroll
-    for (int j = 0; j < DPL; ++j) num[j] = 0.f;
-#pragma unroll
-    for (int s = 0; s < kBatch; ++s) {
-      if (s < ns) {  // same order of additions as the loops below
-        const float wgt = fast_exp2(m_s[s] - ms);
-        den += l_s[s] * wgt;
-#pragma unroll
-        for (int j = 0; j < DPL; ++j) num[j] += acc_s[s][j] * wgt;
-      }
-    }
-    const float lse_nat = ns > 0 ? (mn + log2f(den)) * kLn2 : -INFINITY;
-#pragma unroll
-    for (int j = 0; j < DPL; ++j) {
-      const int d = threadIdx.x + j * 64;
-      if (d >= D) continue;
-      const float o = ns > 0 ? num[j] / den : 0.f;
-      E::store(a.out + b * a.os_b + hq * a.os_h + d * sizeof(typename E::type), sink_gate<E>(o, lse_nat, a.sinks, hq));
-    }
-    if (threadIdx.x == 0) a.lse[static_cast<int64_t>(b) * a.Hq + hq] = lse_nat;
-    return;
-  }
-
-  // More splits than one batch (launches over long contexts): the same lane keeps a running (maximum,
-  // denominator, numerator) over batches of kBatch splits, every load of a batch requested at once.  The
-  // wide variant of this kernel spreads the batches over several wavefronts.
+  // The same lane keeps a running (maximum, denominator, numerator) over batches of kBatch splits, every load
+  // of a batch requested at once.  The wide variant of this kernel spreads the batches over several wavefronts.
   float m_run = -INFINITY, den = 0.f, num[DPL];
 #pragma unroll
   for (int j = 0; j < DPL; ++j) num[j] = 0.f;
-  merge_batches<D, kBatch>(a, p0, 0, kBatch, ns, m_run, den, num);
+  if (ns > 0) fold_batch<D, kBatch>(first, 0, ns, m_run, den, num);
+  merge_batches<D, kBatch>(a, p0, kBatch, kBatch, ns, m_run, den, num);
   finish_merge<E, D>(a, b, hq, ns > 0, m_run, den, num);
 }
 
@@ -787,8 +772,13 @@ __global__ __launch_bounds__(kMergeWideWaves * 64) void paged_decode_merge_wide_
   const int64_t p0 = (static_cast<int64_t>(b) * a.Hq + hq) * a.n_splits;
   __shared__ float s_m[kMergeWideWaves], s_den[kMergeWideWaves], s_num[kMergeWideWaves][DPL * 64];
 
+  // The kernel is a chain of memory latencies: the position of the sequence and this wavefront's first batch of
+  // partial rows are requested together (the batch by the launch's split count; what the sequence does not
+  // have is dropped once its length is known), the later batches of a launch of more than 64 splits after it.
   int64_t L = fp::load_index(a.input_pos, b, a.pos_i64) + 1;
   const int64_t trow = a.batch_idx[b];
+  SplitBatch<D, kBatch> first;
+  load_batch<D, kBatch>(a, p0, wave * kBatch, a.n_splits, 1, first);
   if (trow < 0 || trow >= a.max_batch) L = 0;
   if (L > a.max_context) L = a.max_context;
   const int part = split_part(static_cast<int>(L), a.split_tokens);
@@ -797,7 +787,8 @@ __global__ __launch_bounds__(kMergeWideWaves * 64) void paged_decode_merge_wide_
   float m_run = -INFINITY, den = 0.f, num[DPL];
 #pragma unroll
   for (int j = 0; j < DPL; ++j) num[j] = 0.f;
-  merge_batches<D, kBatch>(a, p0, wave * kBatch, kMergeWideWaves * kBatch, ns, m_run, den, num);
+  if (wave * kBatch < ns) fold_batch<D, kBatch>(first, wave * kBatch, ns, m_run, den, num);
+  merge_batches<D, kBatch>(a, p0, (wave + kMergeWideWaves) * kBatch, kMergeWideWaves * kBatch, ns, m_run, den, num);
   if (lane == 0) {
     s_m[wave] = m_run;
     s_den[wave] = den;
