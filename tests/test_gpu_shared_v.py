@@ -121,10 +121,12 @@ def test_shared_v_and_sink_gate_through_the_even_cut():
     assert not f64(out)[0].any() and np.isneginf(f64(lse)[0]).all()  # the sequence without keys
 
 
-def test_a_cache_that_knows_its_v_copies_decodes_through_the_reference_call():
+@pytest.mark.parametrize("fused", [False, True], ids=["append-launch", "append-in-attention"])
+def test_a_cache_that_knows_its_v_copies_decodes_through_the_reference_call(fused):
     """`install(kv_rep=2)` gives every new cache kv_rep = 2; the unchanged call sequence of the reference
     (insert_kv with expanded K/V, compiled_flex_attn_decode on the returned pool views) then reads V once per
-    group and returns what the plain read returns."""
+    group and returns what the plain read returns -- also when the append is left to the attention launch, which
+    then writes every copy of the new V row."""
     from torch.nn.attention.flex_attention import AuxRequest
 
     from falcon_perception_amd import attention as A
@@ -133,6 +135,7 @@ def test_a_cache_that_knows_its_v_copies_decodes_through_the_reference_call():
     lens = [5, 64, 300, 31]
     st, Hq = expanded_state(57, rep, dtype, P, lens)
     cache = st.cache
+    cache.fuse_decode_append = fused
     B = len(lens)
     bidx = torch.tensor(st.slots, dtype=torch.int64, device=DEV)
     pos = torch.tensor(lens, dtype=torch.int32, device=DEV)
@@ -145,7 +148,9 @@ def test_a_cache_that_knows_its_v_copies_decodes_through_the_reference_call():
     for r in (1, rep):
         cache.kv_rep = r
         K, V = cache.insert_kv(0, k, v, input_pos=pos.view(B, 1), batch_idx=bidx)
+        assert (cache.last_decode_step.k_new is not None) == fused
         out, aux = A.compiled_flex_attn_decode(q, K, V, block_mask=mask, return_aux=AuxRequest(lse=True))
+        assert cache.last_decode_step.k_new is None
         results[r] = (out.clone(), aux.lse.clone())
     assert cache.v_copies_are_identical()
     assert torch.equal(results[1][0], results[rep][0]) and torch.equal(results[1][1], results[rep][1])
