@@ -67,7 +67,25 @@ struct DecodeArgs {
   int64_t kn_b, kn_h, vn_b, vn_h;  // bytes
   int B;         // sequences of the launch
   int n_chunks;  // even cut (kFlat): workgroups per cache head
+  int* plan;     // optional: the step's plan of the even cut (fp_paged_decode_plan), kPlanInts ints per chunk
 };
+
+// The plan of a decode step: what every workgroup of the even cut needs before it can ask for its first K row,
+// computed once per step instead of once per layer and workgroup.  Per chunk (workgroup of a cache head):
+//   rec[0]            pieces of the chunk, or -1: no plan for this chunk (more pieces or pages than a record
+//                     holds), the workgroup works everything out itself
+//   rec[1 .. 3]       B, n_chunks, max_context of the launch the plan was made for: a workgroup that finds other
+//                     values ignores the plan
+//   rec[4 + 6 k ..]   piece k: sequence, first token, tokens, raw length (position + 1), row of the page table
+//                     (-1: not a valid slot), offset of its page ids in the chunk's list
+//   pages[..]         page ids of the pieces, piece after piece (unmapped or foreign pages as 0, like the kernel
+//                     stages them)
+// The positions, the slots and the page table must not change between the plan and the launches that use it.
+constexpr int kPlanPieces = 20;
+constexpr int kPlanRec = 128;            // 4 + 6 * kPlanPieces, rounded up
+constexpr int kPlanPages = kMaxSplitPages;
+constexpr int kPlanInts = kPlanRec + kPlanPages;
+static_assert(4 + 6 * kPlanPieces <= kPlanRec, "a record holds its pieces");
 
 // ---- element access: 16 bytes of a row -----------------------------------
 // A lane holds 16 bytes of a K or V row as four 32-bit words.  `Q` is the lane's
@@ -362,9 +380,10 @@ __global__ __launch_bounds__(kThreads, (decode_waves_per_simd<E, D, G, kPerHeadK
   // Tokens [t0, t0 + part) of sequence b; a partial result goes to row hq * part_mul + part_add of the
   // workspace.
   auto piece = [&](const int b, const int t0, const int part, const bool first, const int64_t part_mul,
-                   const int64_t part_add) {
-  int64_t L = fp::load_index(a.input_pos, b, a.pos_i64) + 1;
-  const int64_t trow = a.batch_idx[b];
+                   const int64_t part_add, const int* pre = nullptr, const int* pre_pages = nullptr) {
+  int64_t L = pre ? static_cast<int64_t>(pre[3]) : fp::load_index(a.input_pos, b, a.pos_i64) + 1;
+  const int64_t trow = pre ? static_cast<int64_t>(pre[4]) : a.batch_idx[b];
+  const int* pages_lds = pre_pages ? pre_pages : s_pages;
   if (trow < 0 || trow >= a.max_batch) L = 0;
   // A position at or beyond max_context is outside what the launch was sized for: the context is read
   // up to max_context from the pool, and the fresh row of a fused append is neither folded nor stored
@@ -420,7 +439,7 @@ __global__ __launch_bounds__(kThreads, (decode_waves_per_simd<E, D, G, kPerHeadK
     a.pd.split(t0, blk0, off_unused);
     int64_t blk_last;
     a.pd.split(t1 - 1, blk_last, off_unused);
-    const int nblk = static_cast<int>(blk_last - blk0) + 1;
+    const int nblk = pre_pages ? 0 : static_cast<int>(blk_last - blk0) + 1;
     for (int i = tid; i < nblk; i += kThreads) {
       int64_t page = 0;
       if (blk0 + i < a.n_pages) page = a.page_table[trow * a.pt_row_stride + blk0 + i];
@@ -436,7 +455,7 @@ __global__ __launch_bounds__(kThreads, (decode_waves_per_simd<E, D, G, kPerHeadK
     v4u kreg[GK][U], vreg[U];
     if (kAligned) {
       // the CH rows of this iteration lie in one page: one base, constant offsets
-      const int page = s_pages[(c0 >> a.pd.shift) - static_cast<int>(blk0)];
+      const int page = pages_lds[(c0 >> a.pd.shift) - static_cast<int>(blk0)];
       const int64_t slot = static_cast<int64_t>(page) * a.pd.page_size + (c0 & (a.pd.page_size - 1)) + grp;
       const char* kp = kbase + slot * ROWB;
       const char* vp = vbase + slot * ROWB;
@@ -454,7 +473,7 @@ __global__ __launch_bounds__(kThreads, (decode_waves_per_simd<E, D, G, kPerHeadK
         int64_t blk;
         int off;
         a.pd.split(t, blk, off);
-        const int64_t slot = static_cast<int64_t>(s_pages[blk - blk0]) * a.pd.page_size + off;
+        const int64_t slot = static_cast<int64_t>(pages_lds[blk - blk0]) * a.pd.page_size + off;
 #pragma unroll
         for (int gk = 0; gk < GK; ++gk) kreg[gk][u] = stream_load(kbase + gk * head_stride + slot * ROWB);
         vreg[u] = stream_load(vbase + slot * ROWB);
@@ -486,7 +505,7 @@ __global__ __launch_bounds__(kThreads, (decode_waves_per_simd<E, D, G, kPerHeadK
       int64_t blk;
       int off;
       a.pd.split(t1 - 1, blk, off);
-      const int64_t slot = static_cast<int64_t>(s_pages[blk - blk0]) * a.pd.page_size + off;
+      const int64_t slot = static_cast<int64_t>(pages_lds[blk - blk0]) * a.pd.page_size + off;
 #pragma unroll
       for (int gk = 0; gk < GK; ++gk) {
         // every cached head gets its K row; V is written to every copy so the pool stays what the
@@ -576,6 +595,37 @@ __global__ __launch_bounds__(kThreads, (decode_waves_per_simd<E, D, G, kPerHeadK
   } else {
     // grid (Hc, n_chunks): every workgroup streams the same number of rows, whatever the lengths are
     __shared__ int s_start[kFlatMaxB + 1];
+    if (a.plan) {
+      // the chunk's record goes where the sequence starts would go, its page ids where a piece stages its own:
+      // one trip to memory instead of positions -> cut -> page table
+      const int* src = a.plan + static_cast<int64_t>(blockIdx.y) * kPlanInts;
+      if (tid < kPlanRec) s_start[tid] = src[tid];
+      s_pages[tid] = src[kPlanRec + tid];  // the first kThreads page ids; more only for very long chunks
+      __syncthreads();
+      const int n = s_start[0];
+      if (n >= 0 && n <= kPlanPieces && s_start[1] == a.B && s_start[2] == a.n_chunks && s_start[3] == a.max_context) {
+        int n_pages_used = 0;
+        if (n > 0) {
+          const int* last = s_start + 4 + 6 * (n - 1);
+          n_pages_used = last[5] + last[2] / a.pd.page_size + 2;  // an upper bound of the list's length
+        }
+        if (n_pages_used > kThreads) {
+          for (int i = kThreads + tid; i < n_pages_used && i < kPlanPages; i += kThreads) s_pages[i] = src[kPlanRec + i];
+          __syncthreads();
+        }
+        const int c = blockIdx.y;
+        // the records are read from registers of a copy: a piece reuses s_start's LDS for nothing, but keeps s_pages
+        for (int k = 0; k < n; ++k) {
+          int r[6];
+#pragma unroll
+          for (int j = 0; j < 6; ++j) r[j] = s_start[4 + 6 * k + j];
+          piece(r[0], r[1], r[2], false, 1, static_cast<int64_t>(c + r[0]) * a.Hq, r, s_pages + r[5]);
+          __syncthreads();  // the LDS of the piece is free again
+        }
+        return;
+      }
+      __syncthreads();  // no usable plan: s_start and s_pages are written anew below
+    }
     flat_starts(a, s_start);
     __syncthreads();
     const int total = s_start[a.B];
@@ -602,6 +652,90 @@ __global__ __launch_bounds__(kThreads, (decode_waves_per_simd<E, D, G, kPerHeadK
       piece(b, t0, t1 - t0, false, 1, static_cast<int64_t>(c + b) * a.Hq);
       __syncthreads();  // the LDS of the piece is free again
     }
+  }
+}
+
+// Writes the plan of a step (see kPlanInts): one wavefront per chunk of the even cut repeats the cut the
+// main kernel would make and looks the page ids of its pieces up.
+__global__ __launch_bounds__(64) void paged_decode_plan_kernel(const DecodeArgs a) {
+  __shared__ int s_start[kFlatMaxB + 1];
+  flat_starts(a, s_start);
+  __syncthreads();
+  const int c = blockIdx.x;
+  int* rec = a.plan + static_cast<int64_t>(c) * kPlanInts;
+  int* pages = rec + kPlanRec;
+  const int total = s_start[a.B];
+  const int len = flat_chunk_len(total, a.n_chunks);
+  const int64_t lo = static_cast<int64_t>(c) * len;
+  const int64_t hi = lo + len < total ? lo + len : total;
+  const int lane = threadIdx.x;
+  const int64_t pool_pages = a.n_slots / a.pd.page_size;
+  int n = 0, page_off = 0;
+  bool ok = true;
+  if (lo < total) {
+    int b = 0;  // first sequence that ends after lo
+    {
+      int left = 0, right = a.B - 1;
+      while (left < right) {
+        const int mid = (left + right) >> 1;
+        if (s_start[mid + 1] > lo) right = mid; else left = mid + 1;
+      }
+      b = left;
+    }
+    for (; b < a.B && s_start[b] < hi; ++b) {
+      const int begin = s_start[b], end = s_start[b + 1];
+      if (end == begin) continue;
+      const int t0 = lo > begin ? static_cast<int>(lo - begin) : 0;
+      const int part = static_cast<int>((hi < end ? hi : end) - begin) - t0;
+      int64_t L = fp::load_index(a.input_pos, b, a.pos_i64) + 1;
+      int64_t trow = a.batch_idx[b];
+      const int64_t L_raw = L > INT32_MAX ? INT32_MAX : L < INT32_MIN ? INT32_MIN : L;
+      if (trow < 0 || trow >= a.max_batch) {
+        trow = -1;
+        L = 0;
+      }
+      if (L > a.max_context) L = a.max_context;
+      if (n >= kPlanPieces) {
+        ok = false;
+        break;
+      }
+      int nblk = 0;
+      if (t0 < L) {  // the pages of tokens t0 .. min(L, t0 + part) - 1, as the main kernel stages them
+        const int t1 = static_cast<int>(L < t0 + part ? L : t0 + part);
+        int64_t blk0, blk_last;
+        int off_unused;
+        a.pd.split(t0, blk0, off_unused);
+        a.pd.split(t1 - 1, blk_last, off_unused);
+        nblk = static_cast<int>(blk_last - blk0) + 1;
+        if (page_off + nblk > kPlanPages) {
+          ok = false;
+          break;
+        }
+        for (int i = lane; i < nblk; i += 64) {
+          int64_t page = 0;
+          if (blk0 + i < a.n_pages) page = a.page_table[trow * a.pt_row_stride + blk0 + i];
+          if (page < 0 || page >= pool_pages) page = 0;  // not a page of the pool
+          pages[page_off + i] = static_cast<int>(page);
+        }
+      }
+      if (lane == 0) {
+        int* r = rec + 4 + 6 * n;
+        r[0] = b;
+        r[1] = t0;
+        r[2] = part;
+        r[3] = static_cast<int>(L_raw);
+        r[4] = static_cast<int>(trow);
+        r[5] = page_off;
+      }
+      page_off += nblk;
+      ++n;
+    }
+  }
+  if (lane == 0) {
+    rec[0] = ok ? n : -1;
+    rec[1] = a.B;
+    rec[2] = a.n_chunks;
+    rec[3] = a.max_context;
   }
 }
 
@@ -816,6 +950,7 @@ __global__ __launch_bounds__(kMergeWideWaves * 64) void paged_decode_merge_wide_
 
 constexpr int kPhasePartial = 1;
 constexpr int kPhaseMerge = 2;
+constexpr int kPhasePlan = 4;  // alone: write the step's plan instead of launching the passes
 
 // Workgroups of the even-cut kernel the current device holds at once (asked once per kernel and device).
 template <typename E, int D, int G, bool kAligned, bool kPerHeadK>
@@ -843,7 +978,7 @@ void launch_decode(const DecodeArgs& a, int B, int phases, hipStream_t st) {
   const bool aligned = a.pd.shift >= 0 && a.pd.page_size % chunk_rows == 0;
   if (a.n_splits == 1) {
     // one split covers every context: the partial pass writes out and lse itself
-    if (!(phases & kPhasePartial)) return;
+    if (!(phases & kPhasePartial)) return;  // also the plan phase: such a launch has no even cut
     if (aligned)
       hipLaunchKernelGGL((paged_decode_kernel<E, D, G, true, true, kPerHeadK>), grid, dim3(kThreads), 0, st, a);
     else
@@ -875,6 +1010,11 @@ void launch_decode(const DecodeArgs& a, int B, int phases, hipStream_t st) {
     DecodeArgs af = a;
     af.B = B;
     af.n_chunks = n_chunks;
+    if (phases & kPhasePlan) {
+      // the plan of a step serves the even cut only; a launch that goes split by split needs none
+      if (a.plan && n_chunks > 0) hipLaunchKernelGGL(paged_decode_plan_kernel, dim3(n_chunks), dim3(64), 0, st, af);
+      return;
+    }
     if (phases & kPhasePartial) {
       if (n_chunks > 0) {
         if (aligned)
@@ -964,6 +1104,9 @@ extern "C" int64_t fp_paged_decode_workspace_bytes(int32_t B, int32_t Hq, int32_
 
 namespace {
 
+// A plan has a record per chunk of the even cut; a launch has at most two chunks per CU and cache head.
+int64_t plan_buffer_bytes() { return 2LL * fp::compute_units() * kPlanInts * static_cast<int64_t>(sizeof(int)); }
+
 struct NewRows {
   const void* k;
   const void* v;
@@ -977,7 +1120,8 @@ int decode_entry(int phases, const NewRows* fresh, const void* q, int64_t q_stri
                  void* workspace, int64_t workspace_bytes, int32_t B, int32_t Hq, int32_t Hc, int32_t kv_rep,
                  int32_t D, int32_t page_size, int32_t n_pages, int32_t max_batch,
                  int64_t n_slots, int32_t max_context, int32_t split_tokens, float scale,
-                 int dtype, void* stream) {
+                 int dtype, void* plan, int64_t plan_bytes, void* stream) {
+  const bool plan_only = phases == kPhasePlan;  // q, out, lse and the workspace are not touched then
   const int eb = fp::elem_bytes(dtype);
   if (eb == 0) return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_decode: unknown dtype %d", dtype);
   if (B < 0 || Hq <= 0 || Hc <= 0 || D <= 0 || page_size <= 0 || n_pages <= 0 || max_batch <= 0 ||
@@ -999,12 +1143,19 @@ int decode_entry(int phases, const NewRows* fresh, const void* q, int64_t q_stri
   if (B > 65535 || Hc > 65535 || Hq > 65535)
     return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_decode: B, Hq or Hc exceeds 65535");
   if (B == 0) return FP_OK;
-  if (!q || !pool_k || !pool_v || !page_table || !batch_idx || !input_pos || !out || !lse)
-    return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: null pointer");
-  if (!fp::aligned(q, 16) || !fp::aligned(pool_k, 16) || !fp::aligned(pool_v, 16) ||
-      (q_stride_b * eb) % 16 || (q_stride_h * eb) % 16)
-    return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: q and pool rows must be 16-byte aligned");
-  if (!fp::aligned(out, eb)) return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: out misaligned");
+  if (!page_table || !batch_idx || !input_pos) return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: null pointer");
+  if (plan_only) {
+    if (!plan) return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode_plan: null plan");
+  } else {
+    if (!q || !pool_k || !pool_v || !out || !lse) return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: null pointer");
+    if (!fp::aligned(q, 16) || !fp::aligned(pool_k, 16) || !fp::aligned(pool_v, 16) ||
+        (q_stride_b * eb) % 16 || (q_stride_h * eb) % 16)
+      return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: q and pool rows must be 16-byte aligned");
+    if (!fp::aligned(out, eb)) return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: out misaligned");
+  }
+  if (plan && (!fp::aligned(plan, 4) || plan_bytes < plan_buffer_bytes()))
+    return fp::fail(FP_ERR_WORKSPACE, "fp_paged_decode: the plan buffer needs %lld bytes (fp_paged_decode_plan_bytes), %lld given",
+                    static_cast<long long>(plan_buffer_bytes()), static_cast<long long>(plan_bytes));
 
   if (split_tokens == 0) split_tokens = default_split_tokens(B, wg_heads, max_context, page_size);
   if (split_tokens % 64) return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode: split_tokens must be a multiple of 64");
@@ -1020,7 +1171,7 @@ int decode_entry(int phases, const NewRows* fresh, const void* q, int64_t q_stri
                static_cast<char*>(out), out_stride_b * eb, out_stride_h * eb, lse, sinks,
                nullptr, nullptr, Hq, wg_heads, fp::PageDiv(page_size), n_pages, max_batch, n_slots,
                max_context, split_tokens, ns, scale * kLog2e,  // scores are kept in log2 units
-               nullptr, nullptr, 0, 0, 0, 0, B, 0};
+               nullptr, nullptr, 0, 0, 0, 0, B, 0, static_cast<int*>(plan)};
   if (fresh) {
     if (!fresh->k || !fresh->v) return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_decode_append: null k_new / v_new");
     if (!fp::aligned(fresh->k, 16) || !fp::aligned(fresh->v, 16) || (fresh->k_stride_b * eb) % 16 ||
@@ -1033,7 +1184,7 @@ int decode_entry(int phases, const NewRows* fresh, const void* q, int64_t q_stri
     a.vn_b = fresh->v_stride_b * eb;
     a.vn_h = fresh->v_stride_h * eb;
   }
-  if (ns > 1) {
+  if (ns > 1 && !plan_only) {
     const int64_t need = static_cast<int64_t>(B) * Hq * ns * (D + 2) * static_cast<int64_t>(sizeof(float));
     if (!workspace || workspace_bytes < need || !fp::aligned(workspace, 16))
       return fp::fail(FP_ERR_WORKSPACE, "fp_paged_decode: workspace of %lld bytes needed, %lld given",
@@ -1063,12 +1214,14 @@ int decode_entry(int phases, const NewRows* fresh, const void* q, int64_t q_stri
       void *workspace, int64_t workspace_bytes, int32_t B, int32_t Hq, int32_t Hc, int32_t kv_rep,        \
       int32_t D,                                                                                          \
       int32_t page_size, int32_t n_pages, int32_t max_batch, int64_t n_slots, int32_t max_context,        \
-      int32_t split_tokens, float scale, int dtype, void *stream
+      int32_t split_tokens, float scale, int dtype, void *plan, int64_t plan_bytes, void *stream
 #define FP_DECODE_ARGS                                                                                     \
   q, q_stride_b, q_stride_h, pool_k, pool_v, page_table, pt_row_stride, batch_idx, input_pos,             \
       pos_index_type, out, out_stride_b, out_stride_h, lse, sinks, workspace, workspace_bytes, B, Hq, Hc, kv_rep, D, \
-      page_size, n_pages, max_batch, n_slots, max_context, split_tokens, scale, dtype, stream
+      page_size, n_pages, max_batch, n_slots, max_context, split_tokens, scale, dtype, plan, plan_bytes, stream
 
+extern "C" int64_t fp_paged_decode_plan_bytes(void) { return plan_buffer_bytes(); }
+extern "C" int fp_paged_decode_plan(FP_DECODE_PARAMS) { return decode_entry(kPhasePlan, nullptr, FP_DECODE_ARGS); }
 extern "C" int fp_paged_decode(FP_DECODE_PARAMS) {
   return decode_entry(kPhasePartial | kPhaseMerge, nullptr, FP_DECODE_ARGS);
 }
@@ -1149,5 +1302,5 @@ extern "C" int fp_paged_decode_noalloc(const void* q, int64_t q_stride_b, int64_
   return decode_entry(kPhasePartial | kPhaseMerge, nullptr, q, q_stride_b, q_stride_h, pool_k, pool_v, page_table,
                       pt_row_stride, batch_idx, input_pos, pos_index_type, out, out_stride_b, out_stride_h, lse, sinks,
                       ws, need ? kScratchBytes : 0, B, Hq, Hc, kv_rep, D, page_size, n_pages, max_batch, n_slots,
-                      max_context, st, scale, dtype, stream);
+                      max_context, st, scale, dtype, nullptr, 0, stream);
 }

@@ -15,7 +15,7 @@ import torch
 _LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib")
 LIB_PATH = os.path.join(_LIB_DIR, "libfp_paged_kv.so")
 
-FP_ABI_VERSION = 5
+FP_ABI_VERSION = 6
 NOALLOC_SCRATCH_BYTES = 64 << 20  # FP_NOALLOC_SCRATCH_BYTES
 FP_DTYPE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
 FP_INDEX = {torch.int32: 0, torch.int64: 1}
@@ -46,8 +46,10 @@ SIGNATURES = {
         c_void_p, c_int64, c_int64, c_void_p, c_void_p,
         c_void_p, c_int64,
         c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
-        c_int64, c_int32, c_int32, c_float, c_int, c_void_p]),
-    "fp_paged_decode_partial": None,  # same signature as fp_paged_decode, filled in below
+        c_int64, c_int32, c_int32, c_float, c_int, c_void_p, c_int64, c_void_p]),
+    "fp_paged_decode_plan_bytes": (c_int64, []),
+    "fp_paged_decode_plan": None,  # same signature as fp_paged_decode, filled in below
+    "fp_paged_decode_partial": None,
     "fp_paged_decode_merge": None,
     "fp_paged_decode_append": None,  # two row pointers and four strides in front of the same list
     "fp_paged_decode_noalloc": None,  # the same list without the workspace pair
@@ -68,10 +70,11 @@ SIGNATURES = {
     "fp_paged_prefill_workspace_bytes": (c_int64, [c_int32, c_int32, c_int32, c_int32, c_int]),
 }
 
+SIGNATURES["fp_paged_decode_plan"] = SIGNATURES["fp_paged_decode"]
 SIGNATURES["fp_paged_decode_partial"] = SIGNATURES["fp_paged_decode"]
 SIGNATURES["fp_paged_decode_merge"] = SIGNATURES["fp_paged_decode"]
 _d = SIGNATURES["fp_paged_decode"][1]
-SIGNATURES["fp_paged_decode_noalloc"] = (c_int, _d[:15] + _d[17:])  # no workspace pointer and size
+SIGNATURES["fp_paged_decode_noalloc"] = (c_int, _d[:15] + _d[17:-3] + _d[-1:])  # no workspace and no plan (pointer, size)
 SIGNATURES["fp_paged_decode_append"] = (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64]
                                         + SIGNATURES["fp_paged_decode"][1])
 

@@ -61,6 +61,7 @@ class PagedDecodeMask:
         self.BLOCK_SIZE = logical.BLOCK_SIZE
         self.seq_lengths = (logical.seq_lengths[0], cache.n_pages * cache.page_size)
         self._physical: dict[str, Tensor | None] = {}
+        self._plan_shape = None  # launch shape the cache's decode plan was made for while this mask owned it
 
     @property
     def max_context(self) -> int:
@@ -253,12 +254,19 @@ def compiled_flex_attn_decode(q: Tensor, k: Tensor, v: Tensor, score_mod=None, b
             cache.last_decode_step = step._replace(k_new=None, v_new=None)
         else:
             cache.flush()
-    out, lse = ops.paged_decode(
-        q, pool_k, pool_v, cache.page_table, block_mask.batch_idx, step.input_pos,
-        cache.page_size, block_mask.max_context, scale=scale,
-        workspace=workspace, split_tokens=split_tokens, sinks=sinks, kv_rep=kv_rep,
-        k_new=k_new, v_new=v_new,
-    )
+    # The plan of the step: the reference converts its mask once per step and every layer consumes it
+    # (paged_inference.py:847-848, model.py:689-699); here the first attention call that meets this mask object
+    # has the decode kernel's per-step work done once, and the layers after it start from the result.
+    plan = cache.decode_plan()
+    args = (q, pool_k, pool_v, cache.page_table, block_mask.batch_idx, step.input_pos, cache.page_size,
+            block_mask.max_context)
+    shape = (q.shape[0], q.shape[1], q.shape[3], k.shape[1], kv_rep, split_tokens, step.input_pos.data_ptr())
+    if cache._decode_plan_owner is not block_mask or block_mask._plan_shape != shape:
+        ops.paged_decode(*args, scale=scale, split_tokens=split_tokens, kv_rep=kv_rep, phase="plan", plan=plan)
+        cache._decode_plan_owner = block_mask
+        block_mask._plan_shape = shape
+    out, lse = ops.paged_decode(*args, scale=scale, workspace=workspace, split_tokens=split_tokens, sinks=sinks,
+                                kv_rep=kv_rep, k_new=k_new, v_new=v_new, plan=plan)
     return _result(out, lse, return_aux, return_lse)
 
 

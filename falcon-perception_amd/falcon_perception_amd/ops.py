@@ -186,7 +186,7 @@ def paged_decode(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor, 
                  split_tokens: int = 0, workspace: Tensor | None = None,
                  out: Tensor | None = None, lse: Tensor | None = None, phase: str = "both",
                  k_new: Tensor | None = None, v_new: Tensor | None = None,
-                 sinks: Tensor | None = None, kv_rep: int = 1) -> tuple[Tensor, Tensor]:
+                 sinks: Tensor | None = None, kv_rep: int = 1, plan: Tensor | None = None) -> tuple[Tensor, Tensor]:
     """Single-query paged attention.  q [B, Hq, 1, D]; pools [Hc, N, D]; returns out [B, Hq, 1, D], lse [B, Hq, 1].
 
     `kv_rep` > 1 declares a cache with one head per query head whose V heads are `kv_rep` identical
@@ -198,8 +198,14 @@ def paged_decode(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor, 
     With `k_new`, `v_new` [B, Hc, 1, D] the call is the whole decode step: the rows are appended at
     `input_pos` (as `kv_append` with clamp would) and attended over in the same launch.
 
-    `phase` = "both" (default), "partial" (split-K pass only, results stay in `workspace`) or
-    "merge" (cross-split merge of a previous partial pass with the same arguments)."""
+    `phase` = "both" (default), "partial" (split-K pass only, results stay in `workspace`),
+    "merge" (cross-split merge of a previous partial pass with the same arguments) or "plan" (write the
+    step's plan into `plan` and launch nothing else).
+
+    `plan`: a uint8 tensor of `decode_plan_bytes()` bytes.  Written by a `phase="plan"` call with the
+    arguments of the step (once per step: the positions and page tables of all layers are the same), it lets
+    the workgroups of a large launch start from one load instead of positions -> cut -> page table; results
+    are bit-identical with and without."""
     N.require_cuda(q, pool_k, pool_v, page_table, batch_idx, input_pos, workspace, out, lse)
     B, Hq, Sq, D = q.shape
     if Sq != 1:
@@ -217,18 +223,28 @@ def paged_decode(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor, 
                            f"per sequence of q ({B})")
     if split_tokens == 0:
         split_tokens = decode_split_tokens(B, Hc // kv_rep if kv_rep > 1 else Hc, max_context, page_size)
-    if workspace is None:  # a workspace the caller brings is checked by the library against the launch
+    planning = phase == "plan"  # writes the plan only: no workspace, no results
+    if workspace is None and not planning:  # a workspace the caller brings is checked by the library against the launch
         need = decode_workspace_bytes(B, Hq, D, max_context, split_tokens)
         if need:
             workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
-    if out is None:
+    if out is None and not planning:
         out = torch.empty((B, Hq, 1, D), dtype=q.dtype, device=q.device)
-    if lse is None:
+    if lse is None and not planning:
         lse = torch.empty((B, Hq, 1), dtype=torch.float32, device=q.device)
-    if out.stride(3) != 1 or not lse.is_contiguous() or lse.dtype != torch.float32:
+    if not planning and (out.stride(3) != 1 or not lse.is_contiguous() or lse.dtype != torch.float32):
         raise RuntimeError("out rows must be dense and lse contiguous float32")
     sinks_ptr = _sinks_ptr(sinks, Hq, q.device)
-    entry = {"both": "fp_paged_decode", "partial": "fp_paged_decode_partial", "merge": "fp_paged_decode_merge"}[phase]
+    entry = {"both": "fp_paged_decode", "partial": "fp_paged_decode_partial", "merge": "fp_paged_decode_merge",
+             "plan": "fp_paged_decode_plan"}[phase]
+    plan_ptr, plan_bytes = None, 0
+    if plan is not None:
+        N.require_cuda(plan)
+        if plan.dtype != torch.uint8 or not plan.is_contiguous():
+            raise RuntimeError("plan must be a contiguous uint8 tensor")
+        plan_ptr, plan_bytes = plan.data_ptr(), plan.numel()
+    elif phase == "plan":
+        raise RuntimeError('phase="plan" needs the plan tensor to write')
     fresh = ()
     if k_new is not None or v_new is not None:
         if phase != "both" or k_new is None or v_new is None:
@@ -244,13 +260,19 @@ def paged_decode(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor, 
         q.data_ptr(), q.stride(0), q.stride(1), pool_k.data_ptr(), pool_v.data_ptr(),
         page_table.data_ptr(), page_table.stride(0), batch_idx.data_ptr(),
         input_pos.data_ptr(), N.index_code(input_pos),
-        out.data_ptr(), out.stride(0), out.stride(1), lse.data_ptr(), sinks_ptr,
+        out.data_ptr() if out is not None else None, out.stride(0) if out is not None else 0,
+        out.stride(1) if out is not None else 0, lse.data_ptr() if lse is not None else None, sinks_ptr,
         workspace.data_ptr() if workspace is not None else None,
         workspace.numel() * workspace.element_size() if workspace is not None else 0,
         B, Hq, Hc, kv_rep, D, page_size, page_table.shape[1], page_table.shape[0],
-        n_slots, max_context, split_tokens, scale, N.dtype_code(q.dtype), N.stream_ptr(q.device))
+        n_slots, max_context, split_tokens, scale, N.dtype_code(q.dtype), plan_ptr, plan_bytes, N.stream_ptr(q.device))
     N.check(rc, entry)
     return out, lse
+
+
+def decode_plan_bytes() -> int:
+    """Bytes a decode plan buffer needs on the current device."""
+    return int(N.lib().fp_paged_decode_plan_bytes())
 
 
 def paged_decode_noalloc(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor, batch_idx: Tensor,

@@ -122,6 +122,8 @@ class PagedKVCache(KVCacheBase):
         self._workspace: Tensor | None = None
         self._retired_workspaces: list[Tensor] = []  # graphs captured earlier still write to these
         self._decode_launch: dict[tuple, tuple[int, int]] = {}
+        self._decode_plan: Tensor | None = None  # the step's plan of the decode kernel (`decode_plan`)
+        self._decode_plan_owner = None           # the mask object it was made for
         self._prefill_workspace: Tensor | None = None
         self._prefill_need: dict[tuple, int] = {}
         # status word of the last prefill mask, on its way to the host (`check_prefill_masks`)
@@ -490,6 +492,14 @@ class PagedKVCache(KVCacheBase):
             hit = (need, self.decode_split_tokens(B, Hc, max_context))
             self._decode_launch[key] = hit
         return (self._workspace if hit[0] else None), hit[1]
+
+    def decode_plan(self) -> Tensor:
+        """Buffer of the decode step's plan (`fp_paged_decode_plan`): allocated once, so that graphs captured
+        with it stay valid.  `compiled_flex_attn_decode` writes it at the first layer of a step and the other
+        layers of the step read it."""
+        if self._decode_plan is None:
+            self._decode_plan = torch.zeros(ops.decode_plan_bytes(), dtype=torch.uint8, device=self._kv.device)
+        return self._decode_plan
 
     def score_bound(self, head_dim: int, scale: float | None) -> float:
         """Bound of |scale * q.k| the prefill kernel may rely on: 0 (unknown) unless q and k are normalised;

@@ -44,7 +44,7 @@
 extern "C" {
 #endif
 
-#define FP_ABI_VERSION 5
+#define FP_ABI_VERSION 6
 
 /* element types of pool / q / k / v */
 #define FP_DTYPE_F32 0
@@ -175,8 +175,42 @@ int64_t fp_paged_decode_workspace_bytes(int32_t B, int32_t Hq, int32_t D,
  *   scale    multiplies q.k (1/sqrt(D) in the reference)
  *   max_context   upper bound of input_pos + 1, fixes the launch grid
  *   split_tokens  tokens per split, a multiple of 64 (0 = library default)
+ *   plan     NULL, or the plan fp_paged_decode_plan wrote for THIS step and launch shape (plan_bytes >=
+ *            fp_paged_decode_plan_bytes()).  Results are bit-identical with and without it.
  * A sequence with input_pos < 0 yields out = 0, lse = -inf.
  */
+int64_t fp_paged_decode_plan_bytes(void);
+
+/*
+ * The plan of a decode step.  The reference converts its block mask once per step
+ * (paged_inference.py:847-848) and every layer's attention consumes it (model.py:689-699); here the
+ * corresponding per-step work is what a workgroup of a large launch (the even cut) has to find out
+ * before it can ask for its first K row: which sequences its chunk covers, their lengths and the page
+ * ids of its rows (positions -> cut -> page table, dependent loads in every workgroup of every layer).
+ * fp_paged_decode_plan does that once, into `plan`; the decode entry points of the same step and the same
+ * shape (B, Hq, Hc, kv_rep, D, page_size, max_context, split_tokens, dtype) then start from one load.
+ * Takes the arguments of the decode call it serves; q, pool_k, pool_v, out, lse and workspace are not
+ * touched and may be NULL.  Between this call and the launches that use the plan, input_pos, batch_idx and the
+ * rows of page_table they name must not change (a workgroup that finds a plan made for another B or
+ * max_context ignores it; stale positions cannot be detected).  A launch that goes split by split (a few
+ * sequences) has no use for a plan: the call then launches nothing and the buffer is ignored.
+ * No counterpart in the reference's kernels; capturable like every other entry point.
+ */
+int fp_paged_decode_plan(const void* q, int64_t q_stride_b, int64_t q_stride_h,
+                         const void* pool_k, const void* pool_v,
+                         const int64_t* page_table, int64_t pt_row_stride,
+                         const int64_t* batch_idx,
+                         const void* input_pos, int pos_index_type,
+                         void* out, int64_t out_stride_b, int64_t out_stride_h,
+                         float* lse, const float* sinks,
+                         void* workspace, int64_t workspace_bytes,
+                         int32_t B, int32_t Hq, int32_t Hc, int32_t kv_rep, int32_t D,
+                         int32_t page_size, int32_t n_pages, int32_t max_batch,
+                         int64_t n_slots, int32_t max_context, int32_t split_tokens,
+                         float scale, int dtype,
+                         void* plan, int64_t plan_bytes,
+                         void* stream);
+
 int fp_paged_decode(const void* q, int64_t q_stride_b, int64_t q_stride_h,
                     const void* pool_k, const void* pool_v,
                     const int64_t* page_table, int64_t pt_row_stride,
@@ -189,6 +223,7 @@ int fp_paged_decode(const void* q, int64_t q_stride_b, int64_t q_stride_h,
                     int32_t page_size, int32_t n_pages, int32_t max_batch,
                     int64_t n_slots, int32_t max_context, int32_t split_tokens,
                     float scale, int dtype,
+                    void* plan, int64_t plan_bytes,
                     void* stream);
 
 /*
@@ -217,6 +252,7 @@ int fp_paged_decode_partial(const void* q, int64_t q_stride_b, int64_t q_stride_
                             int32_t page_size, int32_t n_pages, int32_t max_batch,
                             int64_t n_slots, int32_t max_context, int32_t split_tokens,
                             float scale, int dtype,
+                            void* plan, int64_t plan_bytes,
                             void* stream);
 int fp_paged_decode_merge(const void* q, int64_t q_stride_b, int64_t q_stride_h,
                           const void* pool_k, const void* pool_v,
@@ -230,6 +266,7 @@ int fp_paged_decode_merge(const void* q, int64_t q_stride_b, int64_t q_stride_h,
                           int32_t page_size, int32_t n_pages, int32_t max_batch,
                           int64_t n_slots, int32_t max_context, int32_t split_tokens,
                           float scale, int dtype,
+                          void* plan, int64_t plan_bytes,
                           void* stream);
 
 /*
@@ -261,6 +298,7 @@ int fp_paged_decode_append(const void* k_new, const void* v_new,
                            int32_t page_size, int32_t n_pages, int32_t max_batch,
                            int64_t n_slots, int32_t max_context, int32_t split_tokens,
                            float scale, int dtype,
+                           void* plan, int64_t plan_bytes,
                            void* stream);
 
 /*
