@@ -96,6 +96,9 @@ class DecodeCase:
     workspace: torch.Tensor | None = None
     out: torch.Tensor | None = None
     lse: torch.Tensor | None = None
+    plan: torch.Tensor | None = None  # the step's plan (fp_paged_decode_plan), read by the launches while `planned`
+    planned: bool = True
+    layer_steps: int = 0              # layer-steps run through `run_step` so far
     extra: dict = field(default_factory=dict)
 
     @property
@@ -105,6 +108,28 @@ class DecodeCase:
     @property
     def page_table(self):
         return self.cache.page_table
+
+    @property
+    def _plan(self):
+        return self.plan if self.planned else None
+
+    def make_plan(self):
+        """What a model does once per decode step, before its first layer: positions, slots and page table
+        are those of every layer of the step."""
+        from falcon_perception_amd import ops
+
+        ops.paged_decode(self.q, self.pool_k, self.pool_v, self.cache.page_table, self.batch_idx, self.input_pos,
+                         self.page_size, self.max_context, split_tokens=self.split_tokens, phase="plan",
+                         plan=self.plan, kv_rep=self.cfg.get("kv_rep", 1))
+
+    def run_step(self):
+        """The layer-step at the rate a model of MODEL_LAYERS layers runs it: the plan of the step is written
+        before every MODEL_LAYERS-th layer-step (inside whatever region is being timed), and the fused
+        append + decode launches read it."""
+        if self.planned and self.layer_steps % MODEL_LAYERS == 0:
+            self.make_plan()
+        self.layer_steps += 1
+        return self.run_fused()
 
     @property
     def pool_k(self):
@@ -126,7 +151,8 @@ class DecodeCase:
         return ops.paged_decode(self.q, self.pool_k, self.pool_v, self.cache.page_table, self.batch_idx,
                                 self.input_pos, self.page_size, self.max_context,
                                 split_tokens=self.split_tokens, workspace=self.workspace,
-                                out=self.out, lse=self.lse, phase=phase, kv_rep=self.cfg.get("kv_rep", 1))
+                                out=self.out, lse=self.lse, phase=phase, kv_rep=self.cfg.get("kv_rep", 1),
+                                plan=self._plan)
 
     def run(self):
         self.append()
@@ -140,7 +166,7 @@ class DecodeCase:
                                 self.input_pos, self.page_size, self.max_context,
                                 split_tokens=self.split_tokens, workspace=self.workspace,
                                 out=self.out, lse=self.lse, k_new=self.k_new, v_new=self.v_new,
-                                kv_rep=self.cfg.get("kv_rep", 1))
+                                kv_rep=self.cfg.get("kv_rep", 1), plan=self._plan)
 
     def run_fused_gated(self):
         """run_fused plus the caller's post-attention sink gate (reference model.py:122-127) inside the
@@ -156,7 +182,7 @@ class DecodeCase:
                                 self.input_pos, self.page_size, self.max_context,
                                 split_tokens=self.split_tokens, workspace=self.workspace,
                                 out=out, lse=self.lse, k_new=self.k_new, v_new=self.v_new,
-                                sinks=self.extra["sinks"], kv_rep=self.cfg.get("kv_rep", 1))
+                                sinks=self.extra["sinks"], kv_rep=self.cfg.get("kv_rep", 1), plan=self._plan)
 
     # ---- algorithmic traffic (bytes) --------------------------------------
     def bytes_append(self):
@@ -222,6 +248,8 @@ def make_decode_case(name: str, device="cuda", hbm_budget_gb: float | None = Non
     case.workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=device)
     case.out = torch.empty_like(q)
     case.lse = torch.empty((B, c["Hq"], 1), dtype=torch.float32, device=device)
+    case.plan = torch.zeros(ops.decode_plan_bytes(), dtype=torch.uint8, device=device)
+    case.make_plan()  # launches that are timed alone (events, single-step graphs) read the plan of this step
     return case
 
 
@@ -433,6 +461,16 @@ def graph_ms(fn, steps: int) -> float:
     return statistics.median(regions)
 
 
+def short_kernel_ms(fn, reps: int = 20) -> float:
+    """ms per launch of a kernel too short to time through Python (a library call costs the host about 10 us, and
+    events around it measure that): `reps` launches back to back in one captured graph, replayed."""
+    def many():
+        for _ in range(reps):
+            fn()
+
+    return graph_ms(many, 20) / reps
+
+
 def model_depth_graph_ms(case: "DecodeCase", steps: int, layers: int = MODEL_LAYERS) -> float | None:
     """ms for the fused decode step of ALL layers of the model, replayed from one captured HIP graph: every
     layer has its own K/V planes (the same page table, as in the engine) so nothing is served from cache
@@ -450,11 +488,13 @@ def model_depth_graph_ms(case: "DecodeCase", steps: int, layers: int = MODEL_LAY
         pools[layer, 1].copy_(case.pool_v)
 
     def all_layers():
+        if case.planned:
+            case.make_plan()  # once per step of the model, inside the graph
         for layer in range(layers):
             ops.paged_decode(case.q, pools[layer, 0], pools[layer, 1], case.cache.page_table, case.batch_idx,
                              case.input_pos, case.page_size, case.max_context, split_tokens=case.split_tokens,
                              workspace=case.workspace, out=case.out, lse=case.lse, k_new=case.k_new, v_new=case.v_new,
-                             kv_rep=c.get("kv_rep", 1))
+                             kv_rep=c.get("kv_rep", 1), plan=case._plan)
 
     ms = graph_ms(all_layers, max(steps // 10, 5))
     del pools
@@ -680,7 +720,7 @@ def prefill_drop_in(steps: int = 5, name: str = "cfg3w", layers: int = MODEL_LAY
     return res
 
 
-def decode_drop_in(case: "DecodeCase", steps: int) -> dict:
+def decode_drop_in(case: "DecodeCase", steps: int, model_layers: bool = False) -> dict:
     """The decode layer-step as an unedited engine runs it: `convert_logical_block_mask` once, then `insert_kv` +
     `compiled_flex_attn_decode` (reference paged_inference.py:832-863, model.py:150-162), replayed from a captured
     HIP graph; with the append left to the attention launch (what `install()` switches on) and launched on its own."""
@@ -703,10 +743,12 @@ def decode_drop_in(case: "DecodeCase", steps: int) -> dict:
     saved = (cache.kv_rep, cache.fuse_decode_append)
     cache.kv_rep = case.cfg.get("kv_rep", 1)
 
-    def step():
+    def step(layers=1):
         mask = cache.convert_logical_block_mask(logical, case.batch_idx)
-        K, V = cache.insert_kv(0, case.k_new, case.v_new, input_pos=pos, batch_idx=case.batch_idx)
-        return A.compiled_flex_attn_decode(case.q, K, V, block_mask=mask, return_aux=aux)
+        for _ in range(layers):
+            K, V = cache.insert_kv(0, case.k_new, case.v_new, input_pos=pos, batch_idx=case.batch_idx)
+            res = A.compiled_flex_attn_decode(case.q, K, V, block_mask=mask, return_aux=aux)
+        return res
 
     res = {}
     for fused in (True, False):
@@ -714,6 +756,12 @@ def decode_drop_in(case: "DecodeCase", steps: int) -> dict:
         res["ms_hip_graph_append_in_attention" if fused else "ms_hip_graph_append_launch"] = graph_ms(step, steps)
     cache.fuse_decode_append = True
     res["ms_eager_append_in_attention"] = time_steps(step, steps, 10, samples=7)
+    if model_layers:
+        # A step of the whole model: one mask (and so one plan of the decode launches) for all layers, as the engine
+        # converts its mask once per step.  The layers here share layer 0's planes; a layer streams more bytes than
+        # the last-level cache holds, so no layer is served from what the one before it read.
+        ms = graph_ms(lambda: step(MODEL_LAYERS), max(steps // 10, 5))
+        res["ms_per_layer_hip_graph_of_all_layers"] = ms / MODEL_LAYERS
     cache.kv_rep, cache.fuse_decode_append = saved
     cache.flush()
     return res
@@ -742,7 +790,8 @@ def small_batch_decode(steps: int = 200) -> dict:
     return out
 
 
-def decode_leg(name: str, steps: int = 50, hbm_budget_gb: float | None = None, cpu: bool = False) -> dict:
+def decode_leg(name: str, steps: int = 50, hbm_budget_gb: float | None = None, cpu: bool = False,
+               plan: str = "both") -> dict:
     """One more decode workload next to the headline: the fused step (append inside the split-K pass + merge)
     timed like the headline, the split-K pass alone by events, both priced with the workload's algorithmic
     bytes."""
@@ -753,8 +802,14 @@ def decode_leg(name: str, steps: int = 50, hbm_budget_gb: float | None = None, c
             return {"skipped": f"only {free / 1e9:.0f} GB of HBM free: no room for a long-context pool"}
     case = make_decode_case(name, hbm_budget_gb=hbm_budget_gb)
     c = case.cfg
-    ms_step = time_steps(case.run_fused, steps, 10)
+    case.planned = plan != "off"
+    ms_step = time_steps(case.run_step, steps, 10)
     ms_partial = event_ms(lambda: case.attend("partial"), steps, batch=10)
+    ms_unplanned = None if case.planned else ms_step
+    if plan == "both":
+        case.planned = False
+        ms_unplanned = time_steps(case.run_fused, steps, 10, samples=7)
+        case.planned = True
     alg_decode, alg_append = case.bytes_decode(), case.bytes_append()
     gbps = (alg_decode + alg_append) / (ms_step * 1e-3) / 1e9
     kernel_gbps = alg_decode / (ms_partial * 1e-3) / 1e9
@@ -765,6 +820,7 @@ def decode_leg(name: str, steps: int = 50, hbm_budget_gb: float | None = None, c
                     f"({case.cache.kv_cache.numel() * case.cache.kv_cache.element_size() / 1e9:.1f} GB), contexts "
                     f"{c['prefix']}+U[{c['lo']},{c['hi']}]",
         "ms_per_step": ms_step, "gbps": gbps, "pct_of_hbm_peak": 100.0 * gbps / HBM_PEAK_GBPS,
+        "ms_per_step_without_plan": ms_unplanned,
         "decode_tok_s_per_layer": c["B"] / (ms_step * 1e-3), "algorithmic_bytes": alg_decode + alg_append,
         "roofline": {"bound": "hbm", "kernel": "paged_decode_kernel", "achieved": kernel_gbps, "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": kernel_gbps / HBM_PEAK_GBPS, "ms": ms_partial,
@@ -1028,20 +1084,24 @@ def summary_of(result: dict) -> dict:
     def pct(x):
         return None if x is None else round(100.0 * x, 1)
 
-    out = {"decode_step_us": {}, "decode_step_pct_of_hbm_peak": {}, "decode_kernel_pct_of_hbm_peak": {}}
+    out = {"decode_step_us": {}, "decode_step_without_plan_us": {}, "decode_step_pct_of_hbm_peak": {},
+           "decode_kernel_pct_of_hbm_peak": {}}
     wl = result["config"]["workload"].split(":")[0]
     out["decode_step_us"][wl] = us(result["ms_per_step"])
+    out["decode_step_without_plan_us"][wl] = us(result.get("ms_per_step_without_plan"))
     out["decode_step_pct_of_hbm_peak"][wl] = round(result["pct_of_hbm_peak"], 1)
     out["decode_kernel_pct_of_hbm_peak"][wl] = pct(result["roofline"]["frac"])
     for name, leg in result.get("workloads", {}).items():
         if "ms_per_step" in leg:
             out["decode_step_us"][name] = us(leg["ms_per_step"])
+            out["decode_step_without_plan_us"][name] = us(leg.get("ms_per_step_without_plan"))
             out["decode_step_pct_of_hbm_peak"][name] = round(leg["pct_of_hbm_peak"], 1)
             out["decode_kernel_pct_of_hbm_peak"][name] = pct(leg["roofline"]["frac"])
     out["decode_step_variants_us"] = {
         "separate_append_launch": us(result.get("ms_per_step_separate_append")),
         "sink_gate_in_merge": us(result.get("ms_per_step_with_sink_gate")),
         "hip_graph": us(result.get("ms_per_step_hip_graph")),
+        "plan_kernel": us(result.get("kernels", {}).get("paged_decode_plan_ms")),
         "all_layers_one_graph_per_layer": us(result["ms_all_layers_hip_graph"] / MODEL_LAYERS)
         if result.get("ms_all_layers_hip_graph") else None}
     if "decode_drop_in" in result:
@@ -1103,6 +1163,10 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="cfg2", choices=sorted(DECODE_WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--plan", default="both", choices=["both", "on", "off"],
+                    help="the decode step plan (fp_paged_decode_plan once per %d layer-steps): 'both' times the headline "
+                         "with it and, next to it, without; 'on' / 'off' run every launch of the process one way (for "
+                         "profiling)" % MODEL_LAYERS)
     ap.add_argument("--decode-only", action="store_true",
                     help="only the headline workload: no other configs, no append/gather/prefill measurements")
     ap.add_argument("--pmc-calibration", action="store_true",
@@ -1151,14 +1215,22 @@ def main() -> int:
     case = make_decode_case(args.workload, hbm_budget_gb=args.hbm_budget_gb)
     c = case.cfg
 
-    ms_step = time_steps(case.run_fused, args.steps, args.warmup)
+    case.planned = args.plan != "off"
+    ms_step = time_steps(case.run_step, args.steps, args.warmup)
+    ms_unplanned = ms_partial_unplanned = None
+    if args.plan == "both":
+        case.planned = False  # every launch works its cut out from the positions and the page table itself
+        ms_unplanned = time_steps(case.run_fused, args.steps, args.warmup, samples=7)
+        ms_partial_unplanned = event_ms(lambda: case.attend("partial"), args.steps, batch=10)
+        case.planned = True
+    ms_plan = short_kernel_ms(case.make_plan) if case.planned else None
     ms_separate = time_steps(case.run, args.steps, args.warmup, samples=5)
     ms_gated = time_steps(case.run_fused_gated, args.steps, args.warmup, samples=5)
     ms_graph = graph_ms(case.run_fused, args.steps)
     ms_decode = event_ms(case.attend, args.steps)
     ms_partial = event_ms(lambda: case.attend("partial"), args.steps, batch=10)  # the dominant kernel alone
-    ms_merge = event_ms(lambda: case.attend("merge"), args.steps)
-    ms_append = event_ms(case.append, args.steps)
+    ms_merge = short_kernel_ms(lambda: case.attend("merge"))
+    ms_append = short_kernel_ms(case.append)
     case.attend()
 
     alg_decode = case.bytes_decode()
@@ -1184,14 +1256,19 @@ def main() -> int:
         # measured, not divided: the fused step of all 28 layers (own K/V planes each) in one HIP graph
         "ms_all_layers_hip_graph": None,
         "decode_tok_s_model_measured": None,
-        "step": "fp_paged_decode_append (append fused into the split-K pass) + merge pass",
+        "step": "fp_paged_decode_append (append fused into the split-K pass) + merge pass"
+                + (f"; fp_paged_decode_plan once per {MODEL_LAYERS} layer-steps, inside the timed region (a model plans once "
+                   "per step for all its layers)" if case.planned else "; no step plan"),
+        "ms_per_step_without_plan": ms_unplanned if case.planned else ms_step,
+        "value_without_plan": alg_step / (ms_unplanned * 1e-3) / 1e9 if ms_unplanned else None,
         "ms_per_step_separate_append": ms_separate,
         "ms_per_step_with_sink_gate": ms_gated,  # same step, sigmoid(lse - sink) gate + [B,1,H*D] layout in the merge
         "value_separate_append": alg_step / (ms_separate * 1e-3) / 1e9,
         "ms_per_step_hip_graph": ms_graph,
         "value_hip_graph": alg_step / (ms_graph * 1e-3) / 1e9,
         "kernels": {"paged_decode_ms": ms_decode, "paged_decode_partial_ms": ms_partial,
-                    "paged_decode_merge_ms": ms_merge,
+                    "paged_decode_merge_ms": ms_merge, "paged_decode_plan_ms": ms_plan,
+                    "paged_decode_partial_without_plan_ms": ms_partial_unplanned,
                     "paged_decode_gbps": alg_decode / (ms_decode * 1e-3) / 1e9,
                     "kv_append_ms": ms_append, "kv_append_gbps": alg_append / (ms_append * 1e-3) / 1e9},
         "roofline": {"bound": "hbm", "kernel": "paged_decode_kernel", "achieved": achieved,
@@ -1202,7 +1279,7 @@ def main() -> int:
         result["cpu_baseline"] = cpu_baseline(case)
         result["gpu_over_cpu"] = value / result["cpu_baseline"]["value"]
     if not args.decode_only:
-        result["decode_drop_in"] = decode_drop_in(case, args.steps)
+        result["decode_drop_in"] = decode_drop_in(case, args.steps, model_layers=True)
         ms_model = model_depth_graph_ms(case, args.steps)  # takes and returns 56 GiB
         if ms_model is not None:
             result["ms_all_layers_hip_graph"] = ms_model
@@ -1214,7 +1291,7 @@ def main() -> int:
         for name in ("cfg1", "cfg2x", "cfg2xs", "cfg2d64", "cfg2f32", "cfg4d", "cfg5"):
             if name != args.workload:
                 legs[name] = decode_leg(name, hbm_budget_gb=args.hbm_budget_gb if name == "cfg5" else None,
-                                        cpu=(name == "cfg1" and not args.no_cpu_baseline))
+                                        cpu=(name == "cfg1" and not args.no_cpu_baseline), plan=args.plan)
         result["workloads"] = legs
         result["cfg4_mixed_step"] = cfg4_mixed_step()
         result["prefill_sized"] = append_gather_rates()
