@@ -130,6 +130,49 @@ def test_cfg4_continuous_batching_churn():
         assert len(live) + cache.num_free_pages == n_pages - 1
 
 
+@pytest.mark.parametrize("name", ["cfg2", "cfg2d64", "cfg2f32", "cfg2x", "cfg2xs", "cfg4d"])
+def test_decode_workloads_of_the_bench_at_full_size(name):
+    """The decode workloads bench.py reports (BASELINE configs[1] and its variants: head_dim 64, fp32, the
+    engine's 16-head cache read plainly and with V once per group; the decode part of configs[3]), fused
+    append included: sampled sequences against the float64 oracle, and the step with the step's plan against
+    the step without, bit for bit, pool included."""
+    import bench
+
+    case = bench.make_decode_case(name, device=DEV)
+    c = case.cfg
+    if c.get("kv_rep", 1) > 1:  # the V copies of a group are identical in the engine's cache
+        rep, pv = c["kv_rep"], case.pool_v
+        pv.copy_(pv.view(-1, rep, *pv.shape[1:])[:, :1].expand(-1, rep, *pv.shape[1:]).reshape(pv.shape).clone())
+        case.v_new.copy_(case.v_new.view(c["B"], -1, rep, 1, c["D"])[:, :, :1].expand(-1, -1, rep, -1, -1)
+                         .reshape(case.v_new.shape).clone())
+    before = case.cache.kv_cache.clone()
+    assert case.planned
+    rec = case.plan.view(torch.int32).view(-1, 128 + 1024)[0].cpu()
+    assert rec[0] >= 1 and rec[1] == c["B"]  # the launch is cut evenly and chunk 0 has its record
+    out, lse = (t.clone() for t in case.run_fused())
+    after = case.cache.kv_cache.clone()
+    case.cache.kv_cache.copy_(before)
+    case.planned = False
+    out0, lse0 = case.run_fused()
+    assert torch.equal(out, out0) and torch.equal(lse, lse0)
+    assert torch.equal(case.cache.kv_cache, after)
+    atol, rtol = (2e-5, 2e-5) if case.q.dtype == torch.float32 else (ATOL, RTOL)
+    order = np.argsort(case.lens)
+    for i in [order[0], order[-1], order[len(order) // 2], 0, c["B"] - 1]:
+        slot = int(case.batch_idx[i])
+        eo, el = gathered_oracle_decode(case.q[i], case.pool_k, case.pool_v, case.page_table, slot, case.lens[i] + 1,
+                                        case.page_size)
+        np.testing.assert_allclose(f64(out[i]), eo, atol=atol, rtol=rtol)
+        np.testing.assert_allclose(f64(lse[i]), el, atol=max(atol * 0.1, 1e-5), rtol=rtol)
+        # the appended row is in its slot, bit for bit
+        L = case.lens[i]
+        page = int(case.page_table[slot, L // case.page_size])
+        at = page * case.page_size + L % case.page_size
+        view = torch.int32 if case.q.dtype == torch.float32 else torch.int16
+        assert torch.equal(case.pool_k[:, at].view(view), case.k_new[i, :, 0].view(view))
+        assert torch.equal(case.pool_v[:, at].view(view), case.v_new[i, :, 0].view(view))
+
+
 @pytest.mark.bigmem
 def test_cfg5_long_context_decode_on_a_pool_sized_to_hbm():
     import bench
@@ -141,9 +184,12 @@ def test_cfg5_long_context_decode_on_a_pool_sized_to_hbm():
     case = bench.make_decode_case("cfg5", device=DEV, hbm_budget_gb=budget)
     c = case.cfg
     assert case.pool_k.numel() * 2 > 2**32  # byte offsets inside one plane need 64 bits
-    out, lse = case.run_fused()
+    out, lse = (t.clone() for t in case.run_fused())  # reads the step's plan
     torch.cuda.synchronize()
     assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
+    case.planned = False
+    out0, lse0 = case.run_fused()  # the new rows are in the pool already: the same rows are stored again
+    assert torch.equal(out, out0) and torch.equal(lse, lse0)
     # sampled sequences against the oracle: shortest, longest, and a few in between
     order = np.argsort(case.lens)
     for i in [order[0], order[-1], order[len(order) // 2], 0, c["B"] - 1]:
