@@ -80,12 +80,25 @@ struct DecodeArgs {
 //                     (-1: not a valid slot), offset of its page ids in the chunk's list
 //   pages[..]         page ids of the pieces, piece after piece (unmapped or foreign pages as 0, like the kernel
 //                     stages them)
+//   chunk 0, rec[126]  a hash of the positions and slots the plan was made from (plan_hash_term)
 // The positions, the slots and the page table must not change between the plan and the launches that use it.
+// What the launches do if they did: the merge pass recomputes the hash from the step's positions and slots
+// (it reads them anyway) and stores NaN in every row of out and lse when it differs, so a stale plan fails
+// loudly.  The split-K pass itself does not look (a check of its own position before the fused append's store
+// measured 1.2 us per launch): with a stale plan the fresh rows of the sequences that moved land where the plan
+// says.
 constexpr int kPlanPieces = 20;
+constexpr int kPlanHashAt = 126;
 constexpr int kPlanRec = 128;            // 4 + 6 * kPlanPieces, rounded up
 constexpr int kPlanPages = kMaxSplitPages;
 constexpr int kPlanInts = kPlanRec + kPlanPages;
-static_assert(4 + 6 * kPlanPieces <= kPlanRec, "a record holds its pieces");
+static_assert(4 + 6 * kPlanPieces <= kPlanHashAt && kPlanHashAt < kPlanRec, "a record holds its pieces and the hash");
+
+// Contribution of sequence b to the hash of a step's positions and slots (summed over the sequences, mod 2^32).
+__device__ __forceinline__ uint32_t plan_hash_term(int b, int64_t L, int64_t trow) {
+  const uint32_t w = 2u * static_cast<uint32_t>(b) + 1u;
+  return (static_cast<uint32_t>(L) + static_cast<uint32_t>(trow) * 0x9E3779B1u) * w;
+}
 
 // ---- element access: 16 bytes of a row -----------------------------------
 // A lane holds 16 bytes of a K or V row as four 32-bit words.  `Q` is the lane's
@@ -737,6 +750,14 @@ __global__ __launch_bounds__(64) void paged_decode_plan_kernel(const DecodeArgs 
     rec[2] = a.n_chunks;
     rec[3] = a.max_context;
   }
+  if (c == 0) {
+    uint32_t hash = 0;
+    for (int i = lane; i < a.B; i += 64)
+      hash += plan_hash_term(i, fp::load_index(a.input_pos, i, a.pos_i64) + 1, a.batch_idx[i]);
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) hash += __shfl_xor(hash, off);
+    if (lane == 0) rec[kPlanHashAt] = static_cast<int>(hash);
+  }
 }
 
 // ---- cross-split merge ------------------------------------------------------
@@ -864,9 +885,19 @@ __global__ __launch_bounds__(64) void paged_decode_merge_flat_kernel(const Decod
   const int b = blockIdx.y;
   const int lane = threadIdx.x;
   int before = 0, total = 0, mine = 0;  // rounded lengths: of the sequences before b, of all, of b
+  // the plan's launch values and hash, if the split-K pass had a plan: requested with the positions
+  int planned[4] = {0, 0, 0, 0};
+  if (a.plan) {
+    planned[0] = a.plan[1];
+    planned[1] = a.plan[2];
+    planned[2] = a.plan[3];
+    planned[3] = a.plan[kPlanHashAt];
+  }
+  uint32_t hash = 0;
   for (int i = lane; i < a.B; i += 64) {
     int64_t L = fp::load_index(a.input_pos, i, a.pos_i64) + 1;
     const int64_t trow = a.batch_idx[i];
+    hash += plan_hash_term(i, L, trow);
     if (trow < 0 || trow >= a.max_batch || L < 0) L = 0;
     if (L > a.max_context) L = a.max_context;
     const int Lr = (static_cast<int>(L) + 63) & ~63;
@@ -879,7 +910,11 @@ __global__ __launch_bounds__(64) void paged_decode_merge_flat_kernel(const Decod
     total += __shfl_xor(total, off);
     before += __shfl_xor(before, off);
     mine += __shfl_xor(mine, off);
+    hash += __shfl_xor(hash, off);
   }
+  // the split-K pass followed a plan (same acceptance test as there) that was made from other positions or slots
+  const bool stale = a.plan && planned[0] == a.B && planned[1] == a.n_chunks && planned[2] == a.max_context &&
+                     static_cast<uint32_t>(planned[3]) != hash;
   const int len = flat_chunk_len(total, a.n_chunks);
   const int c_first = before / len;
   const int ns = mine > 0 ? (before + mine - 1) / len - c_first + 1 : 0;
@@ -887,7 +922,8 @@ __global__ __launch_bounds__(64) void paged_decode_merge_flat_kernel(const Decod
 #pragma unroll
   for (int j = 0; j < DPL; ++j) num[j] = 0.f;
   merge_batches<D, 8>(a, static_cast<int64_t>(c_first + b) * a.Hq + hq, 0, 8, ns, m_run, den, num, a.Hq);
-  finish_merge<E, D>(a, b, hq, ns > 0, m_run, den, num);
+  if (stale) den = __builtin_nanf("");  // every row of out and lse: not a result
+  finish_merge<E, D>(a, b, hq, ns > 0 || stale, m_run, den, num);
 }
 
 // Cross-split merge for launches with many splits per sequence: kMergeWideWaves wavefronts per

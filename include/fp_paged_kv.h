@@ -191,8 +191,11 @@ int64_t fp_paged_decode_plan_bytes(void);
  * shape (B, Hq, Hc, kv_rep, D, page_size, max_context, split_tokens, dtype) then start from one load.
  * Takes the arguments of the decode call it serves; q, pool_k, pool_v, out, lse and workspace are not
  * touched and may be NULL.  Between this call and the launches that use the plan, input_pos, batch_idx and the
- * rows of page_table they name must not change (a workgroup that finds a plan made for another B or
- * max_context ignores it; stale positions cannot be detected).  A launch that goes split by split (a few
+ * rows of page_table they name must not change.  A workgroup that finds a plan made for another B or
+ * max_context ignores it.  A plan of the right shape made from other positions or slots is found out by
+ * the merge pass (it reads both anyway and compares a hash of them with the plan's): out and lse are then
+ * NaN in every row, and a fused append has stored the fresh rows of the sequences that moved where the plan
+ * said; changed rows of the page table are not detected.  A launch that goes split by split (a few
  * sequences) has no use for a plan: the call then launches nothing and the buffer is ignored.
  * No counterpart in the reference's kernels; capturable like every other entry point.
  */

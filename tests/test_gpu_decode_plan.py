@@ -121,6 +121,40 @@ def test_a_plan_of_another_launch_and_a_buffer_never_planned_are_ignored():
     assert torch.equal(got_w[0], ref_w[0]) and torch.equal(got_w[1], ref_w[1])
 
 
+def test_a_plan_made_from_other_positions_fails_loudly():
+    """The contract is that positions and slots do not change between the plan and its launches.  If they did
+    (same batch, same shapes, so the workgroups accept the records), the merge pass finds the hash of the
+    step's positions and slots different from the plan's and stores NaN in every row of out and lse."""
+    dtype, B, Hc, G, D, P, split, ctx = torch.bfloat16, 80, 8, 2, 128, 32, 64, 384
+    st = flat_state(98, B, Hc, D, P, ctx - 2, dtype)
+    q = randn(st.gen, (B, Hc * G, 1, D), dtype).to(DEV)
+    pos = torch.tensor(st.lens, dtype=torch.int32, device=DEV)
+    bidx = torch.tensor(st.slots, dtype=torch.int64, device=DEV)
+    kw = dict(max_context=ctx, split_tokens=split)
+    plan = new_plan()
+    decode(st, q, pos, phase="plan", plan=plan, **kw)
+    # one sequence a token further than planned
+    moved = pos.clone()
+    moved[7] += 1
+    out, lse = decode(st, q, moved, plan=plan, **kw)
+    assert torch.isnan(out.float()).all() and torch.isnan(lse).all()
+    # two sequences in each other's slots (the sums of the positions and of the slots are what they were)
+    swapped = bidx.clone()
+    swapped[3], swapped[4] = bidx[4], bidx[3]
+    out, lse = decode(st, q, pos, bidx=swapped, plan=plan, **kw)
+    assert torch.isnan(out.float()).all() and torch.isnan(lse).all()
+    # the passes called separately report it as well
+    ws = torch.empty(ops.decode_workspace_bytes(B, Hc * G, D, ctx, split), dtype=torch.uint8, device=DEV)
+    decode(st, q, moved, workspace=ws, phase="partial", plan=plan, **kw)
+    out, lse = decode(st, q, moved, workspace=ws, phase="merge", plan=plan, **kw)
+    assert torch.isnan(out.float()).all() and torch.isnan(lse).all()
+    # planned anew for what the step holds, the launch is a result again
+    decode(st, q, moved, phase="plan", plan=plan, **kw)
+    out, lse = decode(st, q, moved, plan=plan, **kw)
+    ref = decode(st, q, moved, **kw)
+    assert torch.equal(out, ref[0]) and torch.equal(lse, ref[1])
+
+
 def test_chunks_with_more_pieces_than_a_record_holds_plan_nothing():
     """1024 sequences of at most 64 tokens on 16 cache heads: 32 chunks of about 2000 tokens, 30 pieces each,
     a record holds 20: such chunks are marked -1 and the workgroups cut for themselves."""
