@@ -1063,6 +1063,65 @@ def clock_probe(seconds: float = 2.0) -> dict:
     return out
 
 
+def overlap_probe(iters: int = 2000) -> dict:
+    """`fp_probe_mfma_softmax`: the matrix instructions and the softmax arithmetic of one 64-key tile of the bf16
+    prefill kernel (head_dim 128, score bound), stripped of everything else, alone and in turn, with 1 to 3
+    wavefronts per SIMD, on a quarter of the CUs (the shader clock stays at its maximum there) and on all of them.
+    Reported per slot (one wavefront's tile) and SIMD, in ns and in cycles of the clock read from the driver while
+    the launches run."""
+    from falcon_perception_amd import _native as N
+
+    lib = N.lib()
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    out = torch.empty(cus * 768, dtype=torch.float32, device="cuda")
+    stream = N.stream_ptr(out.device)
+    res = {"what": "ns (cycles) per slot and SIMD; a slot = 32 v_mfma_f32_32x32x16_bf16 + softmax of 32 scores per lane",
+           "iters": iters, "mfma_cycles_at_peak": 32 * 32}
+    for label, wgs in (("quarter_of_the_cus", max(cus // 4, 1)), ("all_cus", cus)):
+        leg = {"workgroups": wgs}
+        for mode, name in ((0, "matrix_only"), (1, "vector_only"), (2, "both_in_turn")):
+            for waves in (1, 2, 3):
+                def launch():
+                    N.check(lib.fp_probe_mfma_softmax(mode, waves, wgs, iters, out.data_ptr(), out.numel(), stream),
+                            "fp_probe_mfma_softmax")
+
+                # launches back to back for about half a second; the clock is read while the second half of them
+                # runs, the time is that of the last ten
+                launch()
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                launch()
+                e1.record()
+                torch.cuda.synchronize()
+                n = max(int(500.0 / max(e0.elapsed_time(e1), 0.05)), 20)
+                marks = [torch.cuda.Event(enable_timing=True) for _ in range(11)]
+                half = torch.cuda.Event()
+                for i in range(n):
+                    if i == n // 2:
+                        half.record()
+                    if i >= n - 10:
+                        marks[i - (n - 10)].record()
+                    launch()
+                marks[10].record()
+                half.synchronize()
+                clocks = []
+                while not marks[10].query():
+                    mhz = shader_clock_mhz()
+                    if mhz:
+                        clocks.append(mhz)
+                    time.sleep(0.002)
+                torch.cuda.synchronize()
+                ms = marks[0].elapsed_time(marks[10]) / 10.0
+                ns = ms * 1e6 / (2.0 * iters * waves)
+                mhz = statistics.median(clocks) if clocks else None
+                leg[f"{name}_{waves}_waves_per_simd"] = {
+                    "ns_per_slot": round(ns, 1), "sclk_mhz": mhz,
+                    "cycles_per_slot": round(ns * mhz / 1e3) if mhz else None}
+        res[label] = leg
+    return res
+
+
 def cpu_model() -> str:
     """Model name of the host processor, as /proc/cpuinfo states it."""
     try:
@@ -1182,6 +1241,9 @@ def main() -> int:
     ap.add_argument("--clock-probe", action="store_true",
                     help="launches of identical prefill workgroups at 32 .. 512 workgroups with the shader clock sampled "
                          "from the driver meanwhile, as JSON")
+    ap.add_argument("--overlap-probe", action="store_true",
+                    help="the matrix and the softmax instructions of one prefill tile, stripped of everything else, alone and "
+                         "in turn with 1 .. 3 wavefronts per SIMD (fp_probe_mfma_softmax), as JSON")
     ap.add_argument("--pieces-only", action="store_true",
                     help="time only KV append, page gather and the fused norm + rotary append at 32768 tokens and print "
                          "their JSON (for profiling)")
@@ -1211,6 +1273,9 @@ def main() -> int:
         return 0
     if args.clock_probe:
         print(json.dumps(clock_probe()))
+        return 0
+    if args.overlap_probe:
+        print(json.dumps(overlap_probe()))
         return 0
     case = make_decode_case(args.workload, hbm_budget_gb=args.hbm_budget_gb)
     c = case.cfg

@@ -70,6 +70,7 @@ SIGNATURES = {
     "fp_paged_prefill_workspace_bytes": (c_int64, [c_int32, c_int32, c_int32, c_int32, c_int]),
 }
 
+SIGNATURES["fp_probe_mfma_softmax"] = (c_int, [c_int, c_int, c_int, c_int, c_void_p, c_int64, c_void_p])
 SIGNATURES["fp_paged_decode_plan"] = SIGNATURES["fp_paged_decode"]
 SIGNATURES["fp_paged_decode_partial"] = SIGNATURES["fp_paged_decode"]
 SIGNATURES["fp_paged_decode_merge"] = SIGNATURES["fp_paged_decode"]

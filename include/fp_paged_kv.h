@@ -450,6 +450,20 @@ int fp_paged_prefill(const void* q, int64_t q_stride_row, int64_t q_stride_h,
                      void* workspace, int64_t workspace_bytes,
                      void* stream);
 
+/*
+ * A measuring kernel, not an operator (no counterpart in the reference; nothing of the attention path calls it):
+ * every wavefront runs 2 * iters times what one wavefront of the bf16 prefill kernel does per 64-key tile at
+ * head_dim 128 with a score bound - 32 v_mfma_f32_32x32x16_bf16 with their K and V operands read from LDS
+ * (mode 0), the softmax of 32 scores per lane: 32 exp2, 32 additions, 16 packs to bf16 (mode 1), or both in
+ * turn (mode 2) - and nothing else: no staging, barrier, mask or address arithmetic.  `workgroups` workgroups of
+ * 256 * waves_per_simd threads (waves_per_simd 1 .. 3; one workgroup fits a CU); `out` takes one float per
+ * launched thread.  Timed by the caller (bench.py --overlap-probe): what it shows is how much of the vector
+ * work a SIMD hides behind the matrix work of another wavefront, which bounds what the prefill kernel's
+ * schedule can reach.
+ */
+int fp_probe_mfma_softmax(int mode, int waves_per_simd, int workgroups, int iters, float* out, int64_t out_floats,
+                          void* stream);
+
 #ifdef __cplusplus
 }
 #endif

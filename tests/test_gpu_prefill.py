@@ -450,3 +450,23 @@ def test_cfg3_chunked_prefill_shape_with_the_score_bound():
         eo, el = O.prefill_attention_paged(f64(case.q[:, :, rows]), pk, pv, case.page_table.cpu().numpy(),
                                            bidx[rows], None, lim[rows], case.page_size)
         assert_close(out[:, :, rows], lse[:, :, rows], eo, el, torch.bfloat16, lse_atol=BOUNDED_LSE_ATOL)
+
+
+def test_the_measuring_kernel_runs_and_refuses_what_it_cannot_launch():
+    """fp_probe_mfma_softmax is a measuring kernel (bench.py --overlap-probe), not an operator: every mode and
+    wavefront count launches and fills its output, bad arguments come back as errors."""
+    from falcon_perception_amd import _native as N
+
+    lib = N.lib()
+    out = torch.full((8 * 768,), float("nan"), dtype=torch.float32, device=DEV)
+    stream = N.stream_ptr(out.device)
+    for mode in (0, 1, 2):
+        for waves in (1, 2, 3):
+            out.fill_(float("nan"))
+            N.check(lib.fp_probe_mfma_softmax(mode, waves, 8, 3, out.data_ptr(), out.numel(), stream), "probe")
+            torch.cuda.synchronize()
+            assert not torch.isnan(out[: 8 * 256 * waves]).any() or mode == 0  # mode 0 accumulates without bound
+            assert torch.isnan(out[8 * 256 * waves:]).all()
+    assert lib.fp_probe_mfma_softmax(2, 4, 8, 3, out.data_ptr(), out.numel(), stream) < 0
+    assert lib.fp_probe_mfma_softmax(3, 1, 8, 3, out.data_ptr(), out.numel(), stream) < 0
+    assert lib.fp_probe_mfma_softmax(2, 3, 9, 3, out.data_ptr(), out.numel(), stream) < 0  # out too small

@@ -414,10 +414,10 @@ def test_only_the_documented_kernels_use_scratch_memory():
     mod = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(mod)
     usage = mod.resource_usage()
-    assert len(usage) > 300  # every template instance of the eight sources
+    assert len(usage) > 300  # every template instance of the nine sources
     for family in ("paged_decode_kernel", "paged_decode_merge", "kv_append_kernel", "kv_gather_kernel", "qkv_rope",
                    "hybrid_row_limits_kernel", "convert_block_ids_kernel", "paged_prefill_kernel", "paged_prefill_f32_kernel",
-                   "paged_prefill_merge_kernel"):
+                   "paged_prefill_merge_kernel", "probe_kernel"):
         assert any(family in name for name in usage), family
     # paged_prefill_kernel<E, 64, G, pow2, 4 wavefronts, bounded>
     allowed = re.compile(r"paged_prefill_kernelINS_\d?(BF16|F16)ELi64ELi\dELb[01]ELi4ELb[01]E")
