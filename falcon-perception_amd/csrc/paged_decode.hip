@@ -1029,7 +1029,9 @@ void launch_decode(const DecodeArgs& a, int B, int phases, hipStream_t st) {
     // 63.9 / 70.6 / 64.2 / 67.9 and 67.2; 16-token pages: 70.0 / 74.4 / 73.9 / 68.9 and 72.6.  fp32 with
     // two chunks per CU: D 128 80.7 against 78.4 split by split, D 64 76.9 against 76.1, 32 q heads 77.4
     // against 73.4 (the even-cut kernels are not held to 128 registers: two workgroups per CU do not need
-    // it, and in fp32 it made them spill).  The even cut needs the lengths of at most kFlatMaxB sequences in LDS, a workspace row per (chunk + sequence),
+    // it, and in fp32 it made them spill).  With the step's plan read by every workgroup the same sweep gives, in us per
+    // step for 1 / 2 / 3 chunks per CU: D 128 110.4 / 111.3 / 112.2; D 64 61.7 / 61.3 / 62.1; page size 64, 32
+    // sequences 89.2 / 90.9 / 90.4: two stays.  The even cut needs the lengths of at most kFlatMaxB sequences in LDS, a workspace row per (chunk + sequence),
     // and chunks within the page-id table.
     int n_chunks = 0;
     {
