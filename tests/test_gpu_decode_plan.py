@@ -98,6 +98,40 @@ def test_a_planned_step_returns_the_bits_of_the_unplanned_one(dtype, D, P, G, re
     np.testing.assert_allclose(f64(lse1), el, atol=max(atol * 0.1, 1e-5), rtol=rtol)
 
 
+@pytest.mark.parametrize("pos_dtype", [torch.int32, torch.int64], ids=str)
+def test_masked_sequences_and_foreign_slots_under_a_plan(pos_dtype):
+    """Sequences the launch must skip - position -1 (a padded row), a slot outside the page table, a position at
+    or beyond max_context - have no piece in the plan either: out 0 / lse -inf for the first two, the context
+    clamped for the third, nothing appended for any of them; bit for bit what the launch without a plan does.
+    Positions as int32 and as int64 (what the engine passes)."""
+    dtype, B, Hc, G, D, P, split, ctx = torch.bfloat16, 80, 8, 2, 128, 32, 64, 384
+    st = flat_state(99, B, Hc, D, P, ctx - 2, dtype)
+    q = randn(st.gen, (B, Hc * G, 1, D), dtype).to(DEV)
+    k_new = randn(st.gen, (B, Hc, 1, D), dtype).to(DEV)
+    v_new = randn(st.gen, (B, Hc, 1, D), dtype).to(DEV)
+    pos = torch.tensor(st.lens, dtype=pos_dtype, device=DEV)
+    bidx = torch.tensor(st.slots, dtype=torch.int64, device=DEV)
+    pos[5] = -1
+    bidx[9] = B + 40      # beyond max_batch
+    bidx[11] = -3
+    pos[13] = ctx + 7     # beyond what the launch was sized for
+    kw = dict(max_context=ctx, split_tokens=split, bidx=bidx)
+    before = st.cache.kv_cache.clone()
+    ref = decode(st, q, pos, k_new=k_new, v_new=v_new, **kw)
+    pool_ref = st.cache.kv_cache.clone()
+    st.cache.kv_cache.copy_(before)
+    plan = new_plan()
+    decode(st, q, pos, phase="plan", plan=plan, **kw)
+    got = decode(st, q, pos, k_new=k_new, v_new=v_new, plan=plan, **kw)
+    assert torch.equal(got[0], ref[0]) and torch.equal(got[1], ref[1])
+    assert torch.equal(st.cache.kv_cache, pool_ref)
+    for i in (5, 9, 11):
+        assert not got[0][i].any() and torch.isneginf(got[1][i]).all()
+    assert torch.isfinite(got[1][13]).all()
+    changed = (pool_ref != before).flatten(0, -3).any(-1)  # per pool slot, any layer / plane / head
+    assert int(changed.sum()) == (B - 4) * 2 * Hc  # one K and one V row per head of every sequence that appended
+
+
 def test_a_plan_of_another_launch_and_a_buffer_never_planned_are_ignored():
     """A workgroup uses a record only if it carries the launch's batch, chunk count and max_context; anything
     else (a plan made for one sequence more, for another max_context, a buffer of zeros or of 0xA5) leaves the
