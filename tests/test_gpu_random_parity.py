@@ -119,7 +119,8 @@ def test_prefill_random(seed):
 def test_decode_random_large_launches(seed):
     """Many sequences and small splits, so that the launch has more workgroups than the GPU holds at once
     (the launch then takes the even cut over the flattened contexts): batch sizes that are no multiple
-    of 64, empty and masked-out sequences, every page size and head grouping of `draw`."""
+    of 64, empty and masked-out sequences, every page size and head grouping of `draw`; odd seeds with the
+    step's plan."""
     rng, P, D, G, Hc, dtype = draw(200 + seed, [torch.bfloat16, torch.float16, torch.float32])
     Hc = int(rng.choice([4, 8]))
     B = int(rng.integers(90, 260))
@@ -140,8 +141,15 @@ def test_decode_random_large_launches(seed):
     pk, pv = st.pool_planes()
     max_ctx = 448
     before = st.cache.kv_cache.clone()
+    plan = None
+    if seed % 2:  # every other configuration through the step's plan (fp_paged_decode_plan)
+        plan = torch.zeros(ops.decode_plan_bytes(), dtype=torch.uint8, device=DEV)
+        ops.paged_decode(q.to(DEV), pk, pv, st.cache.page_table, bidx, pos.to(DEV), P, max_ctx, split_tokens=64,
+                         phase="plan", plan=plan)
+        # (written where the launch is cut evenly; one-token pages with many sequences go split by split: untouched)
+        assert int(plan.view(torch.int32)[1]) in (0, B)
     out, lse = ops.paged_decode(q.to(DEV), pk, pv, st.cache.page_table, bidx, pos.to(DEV), P, max_ctx,
-                                split_tokens=64, k_new=k1.to(DEV), v_new=v1.to(DEV))
+                                split_tokens=64, k_new=k1.to(DEV), v_new=v1.to(DEV), plan=plan)
     keep = [i for i in range(B) if i != masked]
     want = before.cpu().clone()
     wv = want.view(torch.int16 if dtype != torch.float32 else torch.int32).numpy()
