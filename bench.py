@@ -1312,7 +1312,9 @@ def main() -> int:
         "config": {"workload": f"{case.name}: decode layer-step, batch {c['B']}, {c['Hq']} q / {c['Hc']} kv heads, "
                                f"head_dim {c['D']}, page_size {c['P']}, {c['n_pages']}-page pool, contexts "
                                f"{c['prefix']}+U[{c['lo']},{c['hi']}], seed {c['seed']}",
-                   "tokens_in_cache": sum(case.lens), "split_tokens": case.split_tokens},
+                   "tokens_in_cache": sum(case.lens), "split_tokens": case.split_tokens,
+                   "step_plan": (f"fp_paged_decode_plan launched once per {MODEL_LAYERS} layer-steps inside the timed region "
+                                 "(ms_per_step_without_plan: no plan at all)") if case.planned else "none"},
         "timing": "ms_per_step = median of 21 regions of exactly `steps` back-to-back steps, synchronised on both "
                   "sides; kernel times = median of >= 20 HIP-event samples on the launch stream",
         "pct_of_hbm_peak": 100.0 * value / HBM_PEAK_GBPS,
