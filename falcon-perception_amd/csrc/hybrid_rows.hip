@@ -25,9 +25,10 @@
 // One workgroup scans the packed row.  The tokens are first classified with loads that run over the row in
 // memory order (two tokens per lane and step), four bits per token into LDS: how many soi it counts as (its own
 // and a virtual one in front of a declared run), whether it is an eoi, whether its document ends after it.
-// Then each thread owns a contiguous chunk of the classes: the chunk totals are combined with an LDS prefix
-// sum (forward) and an LDS suffix minimum (backward).  L is at most 65536 tokens; 23040 take 29 microseconds
-// and 32768 take 40 (reading the ids chunk by chunk, every lane at its own stride, took 61 for 23040).
+// Then each thread owns a contiguous chunk of the classes: the chunk totals are combined with a prefix sum
+// (forward) and a suffix minimum (backward), inside the wavefronts by lane shifts and over the 16 wavefront totals
+// through LDS; the limits are staged in LDS and leave in memory order.  L is at most 65536 tokens; 23040 take 21
+// microseconds and 32768 take 32 (reading the ids chunk by chunk, every lane at its own stride, took 61 for 23040).
 #include "fp_common.h"
 
 namespace {
@@ -35,6 +36,7 @@ namespace {
 constexpr int kThreads = 1024;
 constexpr int kMaxL = 65536;
 constexpr int kSoiMask = 3, kEoiBit = 4, kRunEndBit = 8;
+constexpr int kSegment = 32768;  // rows whose limits are staged in LDS at a time (as limit - 1, 16 bits: a limit is 1 .. 65536)
 
 __global__ __launch_bounds__(kThreads) void hybrid_row_limits_kernel(const int64_t* __restrict__ ids,
                                                                      const int64_t* __restrict__ docs,
@@ -44,10 +46,11 @@ __global__ __launch_bounds__(kThreads) void hybrid_row_limits_kernel(const int64
                                                                      int32_t* __restrict__ row_hi,
                                                                      int32_t* __restrict__ status) {
   __shared__ uint8_t s_cls[kMaxL / 2];  // two tokens per byte
-  __shared__ int s_soi[kThreads];
-  __shared__ int s_eoi[kThreads];
-  __shared__ int s_next[kThreads];
+  __shared__ int s_soi[kThreads / 64];
+  __shared__ int s_eoi[kThreads / 64];
+  __shared__ int s_next[kThreads / 64];
   __shared__ int s_flags;
+  __shared__ uint16_t s_out[kSegment];
 
   const int tid = threadIdx.x;
   if (tid == 0) s_flags = 0;
@@ -64,20 +67,34 @@ __global__ __launch_bounds__(kThreads) void hybrid_row_limits_kernel(const int64
     }
     return c;
   };
-  for (int i = tid; 2 * i < L; i += kThreads) {
-    const int k0 = 2 * i, k1 = k0 + 1;
-    const bool two = k1 < L;
-    const int64_t id0 = ids[k0], id1 = two ? ids[k1] : 0;
-    int64_t dm = 0, d0 = 0, d1 = 0, d2 = 0;
-    if (docs) {
-      dm = k0 > 0 ? docs[k0 - 1] : 0;
-      d0 = docs[k0];
-      d1 = two ? docs[k1] : 0;
-      d2 = k1 + 1 < L ? docs[k1 + 1] : 0;
+  // kBatch steps of a lane at a time: every load of the batch is requested before the first class is computed
+  // (step by step the loop was a chain of round trips to memory, a dozen of them at 23040 tokens)
+  constexpr int kBatch = 4;
+  for (int i0 = tid; 2 * i0 < L; i0 += kBatch * kThreads) {
+    int64_t id0[kBatch], id1[kBatch], dm[kBatch], d0[kBatch], d1[kBatch], d2[kBatch];
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) {
+      const int k0 = 2 * (i0 + j * kThreads), k1 = k0 + 1;
+      const bool one = k0 < L, two = k1 < L;
+      id0[j] = one ? ids[k0] : 0;
+      id1[j] = two ? ids[k1] : 0;
+      dm[j] = d0[j] = d1[j] = d2[j] = 0;
+      if (docs) {
+        dm[j] = one && k0 > 0 ? docs[k0 - 1] : 0;
+        d0[j] = one ? docs[k0] : 0;
+        d1[j] = two ? docs[k1] : 0;
+        d2[j] = k1 + 1 < L ? docs[k1 + 1] : 0;
+      }
     }
-    int byte = classify(k0, id0, dm, d0, d1);
-    if (two) byte |= classify(k1, id1, d0, d1, d2) << 4;
-    s_cls[i] = static_cast<uint8_t>(byte);
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) {
+      const int i = i0 + j * kThreads;
+      const int k0 = 2 * i, k1 = k0 + 1;
+      if (k0 >= L) break;
+      int byte = classify(k0, id0[j], dm[j], d0[j], d1[j]);
+      if (k1 < L) byte |= classify(k1, id1[j], d0[j], d1[j], d2[j]) << 4;
+      s_cls[i] = static_cast<uint8_t>(byte);
+    }
   }
   __syncthreads();
   auto cls = [&](int k) { return (s_cls[k >> 1] >> ((k & 1) * 4)) & 15; };
@@ -92,20 +109,29 @@ __global__ __launch_bounds__(kThreads) void hybrid_row_limits_kernel(const int64
     n_soi += c & kSoiMask;
     n_eoi += (c & kEoiBit) != 0;
   }
-  s_soi[tid] = n_soi;
-  s_eoi[tid] = n_eoi;
-  __syncthreads();
-  // inclusive prefix sums over the chunk totals
-  for (int d = 1; d < kThreads; d <<= 1) {
-    const int a = tid >= d ? s_soi[tid - d] : 0;
-    const int b = tid >= d ? s_eoi[tid - d] : 0;
-    __syncthreads();
-    s_soi[tid] += a;
-    s_eoi[tid] += b;
-    __syncthreads();
+  // inclusive prefix sums over the chunk totals: inside every wavefront by lane shifts, then over the 16
+  // wavefront totals through LDS (two barriers instead of the twenty of a scan over all 1024 threads)
+  const int lane = tid & 63, wave = tid >> 6;
+  int inc_soi = n_soi, inc_eoi = n_eoi;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int a = __shfl_up(inc_soi, d), b = __shfl_up(inc_eoi, d);
+    if (lane >= d) {
+      inc_soi += a;
+      inc_eoi += b;
+    }
   }
-  const int base_soi = s_soi[tid] - n_soi;  // counts before this chunk
-  const int base_eoi = s_eoi[tid] - n_eoi;
+  if (lane == 63) {
+    s_soi[wave] = inc_soi;
+    s_eoi[wave] = inc_eoi;
+  }
+  __syncthreads();
+  for (int w = 0; w < wave; ++w) {
+    inc_soi += s_soi[w];
+    inc_eoi += s_eoi[w];
+  }
+  const int base_soi = inc_soi - n_soi;  // counts before this chunk
+  const int base_eoi = inc_eoi - n_eoi;
 
   // first index in this chunk that ends a span (not inside, or a soi), L if none
   int first_end = L;
@@ -123,26 +149,37 @@ __global__ __launch_bounds__(kThreads) void hybrid_row_limits_kernel(const int64
     }
   }
   if (flags) atomicOr(&s_flags, flags);
-  s_next[tid] = first_end;
-  __syncthreads();
-  // inclusive suffix minimum over chunks
-  for (int d = 1; d < kThreads; d <<= 1) {
-    const int a = tid + d < kThreads ? s_next[tid + d] : L;
-    __syncthreads();
-    s_next[tid] = min(s_next[tid], a);
-    __syncthreads();
+  // exclusive suffix minimum over chunks (the first span end after this chunk), the same way
+  int suf = first_end;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int a = __shfl_down(suf, d);
+    if (lane + d < 64) suf = min(suf, a);
   }
-  int next_end = tid + 1 < kThreads ? s_next[tid + 1] : L;  // first span end after this chunk
+  if (lane == 0) s_next[wave] = suf;  // minimum of the whole wavefront
+  __syncthreads();
+  int next_end = __shfl_down(suf, 1);  // minimum over the later lanes of this wavefront
+  if (lane == 63) next_end = L;
+  for (int w = wave + 1; w < kThreads / 64; ++w) next_end = min(next_end, s_next[w]);
 
-  // walk the chunk backwards; counts at k are recovered by undoing token k+1
+  // walk the chunk backwards; counts at k are recovered by undoing token k+1.  The limits go to global memory
+  // through LDS, a segment of kSegment rows at a time from the last to the first: written from the chunks they
+  // would leave as 4-byte pieces `per` rows apart, 64 different cache lines per store instruction.
   int o = base_soi + n_soi, c = base_eoi + n_eoi;  // inclusive counts at hi - 1
-  for (int k = hi - 1; k >= lo; --k) {
-    const int cl = cls(k);
-    const bool inside = o - c > 0;
-    row_hi[k] = inside ? next_end : k + 1;
-    if (!inside || (cl & kSoiMask)) next_end = k;
-    o -= cl & kSoiMask;
-    c -= (cl & kEoiBit) != 0;
+  int k = hi - 1;
+  for (int seg_lo = ((L - 1) / kSegment) * kSegment; seg_lo >= 0; seg_lo -= kSegment) {
+    for (; k >= lo && k >= seg_lo; --k) {
+      const int cl = cls(k);
+      const bool inside = o - c > 0;
+      s_out[k - seg_lo] = static_cast<uint16_t>((inside ? next_end : k + 1) - 1);
+      if (!inside || (cl & kSoiMask)) next_end = k;
+      o -= cl & kSoiMask;
+      c -= (cl & kEoiBit) != 0;
+    }
+    __syncthreads();
+    const int n = min(kSegment, L - seg_lo);
+    for (int i = tid; i < n; i += kThreads) row_hi[seg_lo + i] = static_cast<int>(s_out[i]) + 1;
+    __syncthreads();
   }
   if (tid == 0 && status) *status = s_flags;  // every atomicOr lies before the barriers of the suffix scan
 }
