@@ -297,6 +297,10 @@ class PrefillCase:
     score_bound: float = 0.0
     use_bound: bool = True
     input_ids: torch.Tensor | None = None   # [1, Lq] int64 token ids the row limits follow from
+    # the step's query tiles by decreasing key range (fp_paged_prefill_tile_order): made once per step, as the row
+    # limits are, and taken by every layer's launch; only at head_dim 64, where the order of the workgroups matters
+    tile_order: tuple | None = None
+    use_order: bool = True
 
     @property
     def page_size(self):
@@ -325,7 +329,17 @@ class PrefillCase:
                                  self.row_limit, self.page_size,
                                  workspace=self.cache.prefill_workspace(self.q.shape[2], self.q.shape[1], self.q.shape[3],
                                                                         self.pool_k.shape[0], self.q.dtype),
-                                 score_bound=self.score_bound if bounded else 0.0)
+                                 score_bound=self.score_bound if bounded else 0.0,
+                                 tile_order=self.tile_order if self.use_order else None)
+
+    def make_tile_order(self):
+        """What a model does once per prefill step, next to the mask: rank the step's query tiles."""
+        from falcon_perception_amd import ops
+
+        Lq, Hq, D, Hc = self.q.shape[2], self.q.shape[1], self.q.shape[3], self.pool_k.shape[0]
+        ws = self.cache.prefill_workspace(Lq, Hq, D, Hc, self.q.dtype)
+        rows = ops.prefill_tile_rows(Lq, Hq, Hc, D, self.q.dtype, ws.numel() if ws is not False else 0)
+        self.tile_order = ops.prefill_tile_order(self.batch_idx, self.row_limit, rows) if rows else None
 
     def run(self):
         self.append()
@@ -630,9 +644,17 @@ def prefill_rate(steps: int = 10, name: str = "cfg3", bounded: bool = True, both
     case = make_prefill_case(name)
     case.use_bound = bounded
     case.append()
+    ms_order = ms_no_order = None
+    if case.q.shape[3] == 64 and case.q.dtype != torch.float32:
+        case.make_tile_order()
+        ms_order = short_kernel_ms(case.make_tile_order)
     for _ in range(3):
         case.attend()
     ms = event_ms(case.attend, steps, batch=4)
+    if case.tile_order is not None and both:
+        case.use_order = False
+        ms_no_order = event_ms(case.attend, steps, batch=4)
+        case.use_order = True
     ms_a = event_ms(case.append, steps)
     tf = case.flops() / (ms * 1e-3) / 1e12
     ms_unbounded = None
@@ -656,6 +678,11 @@ def prefill_rate(steps: int = 10, name: str = "cfg3", bounded: bool = True, both
            "chunk_append_ms": ms_a, "flops": case.flops(),
            "key_tiles_per_query_tile": {"longest": int(tiles.max()), "mean": round(float(tiles.mean()), 1),
                                         "query_tiles_per_head": int(tiles.numel())}}
+    if ms_order is not None:
+        res["tile_order"] = ("workgroups start longest key range first: fp_paged_prefill_tile_order once per step, outside "
+                             "the timed launch as the row limits are")
+        res["tile_order_kernel_ms"] = ms_order
+        res["paged_prefill_ms_no_tile_order"] = ms_no_order
     if case.q.dtype == torch.float32:
         res["frac_of_f32_mfma_peak"] = tf / MFMA_F32_PEAK_TFLOPS
     else:
@@ -1181,6 +1208,8 @@ def summary_of(result: dict) -> dict:
         pf[name] = {"us": us(leg["paged_prefill_ms"]), "tflops": round(leg["tflops"], 1), "pct_of_mfma_peak": pct(frac)}
         if "paged_prefill_ms_no_score_bound" in leg:
             pf[name]["us_no_score_bound"] = us(leg["paged_prefill_ms_no_score_bound"])
+        if leg.get("paged_prefill_ms_no_tile_order"):
+            pf[name]["us_no_tile_order"] = us(leg["paged_prefill_ms_no_tile_order"])
     if pf:
         out["prefill"] = pf
     if "prefill_drop_in" in result:

@@ -79,6 +79,9 @@ struct PrefillArgs {
   // the bytes of fp32 partials; the merge pass is bound by this traffic), with its maximum and denominator
   short* ws_acc;  // [n_key_splits, Lq, Hq, D] elements of the model dtype
   float* ws_ml;   // [n_key_splits, Lq, Hq, 2]: running maximum (log2 units), denominator
+  // optional (fp_paged_prefill_tile_order): the query tile workgroup row y works on, longest key range first
+  const int* order;
+  int order_rows;  // rows per query tile the order was made for; another tile size ignores it
 };
 
 struct BF16 {
@@ -179,7 +182,14 @@ __global__ __launch_bounds__(W * 64, (W == 4 && D == 64 ? 3 : 2)) void paged_pre
   // linear id = cache head + Hc * tile: all tiles that read one cache head run on the XCD that
   // already holds its K/V in L2
   const int hc = blockIdx.x;
-  const int tile = a.n_tiles - 1 - blockIdx.y;  // longest key ranges first
+  // Workgroups are handed out in the order of their ids, so the ids should run from the longest key range to the
+  // shortest.  Without an order from the caller: descending tile index, which is that inside a sequence (later
+  // rows see more keys) but not across a packed row of several.
+  int tile = a.n_tiles - 1 - blockIdx.y;
+  if (a.order) {
+    tile = a.order[blockIdx.y];
+    tile = tile < 0 ? 0 : tile >= a.n_tiles ? a.n_tiles - 1 : tile;  // whatever the buffer holds, no row outside the launch
+  }
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int hq = hc * G + wave % G;  // query head of this wavefront
@@ -816,10 +826,12 @@ void launch_group(const PrefillArgs& a0, float score_bound, void* workspace, int
     if (shares == 1) {
       constexpr int BM4 = (4 / G) * 32;
       a.n_tiles = (a.Lq + BM4 - 1) / BM4;
+      if (a.order_rows != BM4) a.order = nullptr;
       launch_main<E, D, G, 4>(a, dim3(a.Hc, a.n_tiles, 1), bounded, st);
       return;
     }
   }
+  if (a.order_rows != BM) a.order = nullptr;
   launch_main<E, D, G, kWaves>(a, dim3(a.Hc, a.n_tiles, shares), bounded, st);
   if (shares > 1) {
     const int64_t items = static_cast<int64_t>(a.Lq) * a.Hq;
@@ -839,7 +851,100 @@ int launch(const PrefillArgs& a, float score_bound, void* ws, int64_t ws_bytes, 
   }
 }
 
+// Rows per query tile of the launch fp_paged_prefill makes for this shape with a workspace of this size (the
+// same decisions as launch_group); 0 for the fp32 kernel, which takes no order.
+int tile_rows_for(int Lq, int Hq, int Hc, int D, int dtype, int64_t workspace_bytes) {
+  if (dtype == FP_DTYPE_F32) return 0;
+  const int g = Hq / Hc;
+  const int bm = (kWaves / g) * 32;
+  const int n_tiles = (Lq + bm - 1) / bm;
+  int shares = workspace_bytes > 0 ? key_shares_for(static_cast<int64_t>(Hc) * n_tiles, FP_DTYPE_BF16) : 1;
+  while (shares > 1 && share_bytes(shares, Lq, Hq, D, 2) > workspace_bytes) --shares;
+  return (g <= 4 && D == 64 && shares == 1) ? (4 / g) * 32 : bm;
+}
+
+// Query tiles of a step ordered by the key tiles they walk, longest first.  One workgroup: the largest limit of
+// every tile's rows (padding rows, sequence 0, count as 0), then every tile's rank by counting the
+// tiles that go before it (among equals the later tile first, as in the order the kernel uses by itself).
+constexpr int kOrderThreads = 1024;
+constexpr int kOrderMaxTiles = 4096;
+
+__global__ __launch_bounds__(kOrderThreads) void prefill_tile_order_kernel(const int64_t* __restrict__ batch_idx,
+                                                                           const int32_t* __restrict__ row_limit, int Lq,
+                                                                           int tile_shift, int n_tiles, int* __restrict__ order) {
+  __shared__ __attribute__((aligned(16))) int s_kt[kOrderMaxTiles];
+  const int tid = threadIdx.x;
+  for (int t = tid; t < n_tiles; t += kOrderThreads) s_kt[t] = 0;
+  __syncthreads();
+  // a tile is 32 rows or more and the rows run along the lanes: the lanes of half a wavefront share a tile and
+  // combine their limits by lane exchanges before one of them goes to LDS
+  constexpr int kBatch = 4;  // steps whose loads are requested together
+  for (int r0 = 0; r0 < Lq; r0 += kBatch * kOrderThreads) {
+    int64_t seq[kBatch];
+    int lim[kBatch];
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) {
+      const int r = r0 + j * kOrderThreads + tid;
+      seq[j] = r < Lq ? batch_idx[r] : 0;
+      lim[j] = r < Lq ? row_limit[r] : 0;
+    }
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) {
+      const int r = r0 + j * kOrderThreads + tid;
+      int m = seq[j] != 0 ? lim[j] : 0;
+#pragma unroll
+      for (int off = 1; off < 32; off <<= 1) m = max(m, __shfl_xor(m, off));
+      if ((tid & 31) == 0 && m > 0 && r < Lq) atomicMax(&s_kt[r >> tile_shift], m);
+    }
+  }
+  __syncthreads();
+  const int padded = (n_tiles + 3) & ~3;  // the ranking reads four tiles at a time; -1 goes before nothing
+  for (int t = tid; t < padded; t += kOrderThreads) s_kt[t] = t < n_tiles ? (s_kt[t] + kTileN - 1) / kTileN : -1;
+  __syncthreads();
+  for (int t = tid; t < n_tiles; t += kOrderThreads) {
+    const int mine = s_kt[t];
+    int rank = 0;
+#pragma unroll 4
+    for (int u = 0; u < padded; u += 4) {
+      const int4 o = *reinterpret_cast<const int4*>(&s_kt[u]);
+      rank += (o.x > mine || (o.x == mine && u > t)) + (o.y > mine || (o.y == mine && u + 1 > t)) +
+              (o.z > mine || (o.z == mine && u + 2 > t)) + (o.w > mine || (o.w == mine && u + 3 > t));
+    }
+    order[rank] = t;
+  }
+}
+
 }  // namespace
+
+extern "C" int32_t fp_paged_prefill_tile_rows(int32_t Lq, int32_t Hq, int32_t Hc, int32_t D, int dtype,
+                                              int64_t workspace_bytes) {
+  if (Lq < 0 || Hq <= 0 || Hc <= 0 || Hq % Hc || (D != 64 && D != 128))
+    return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_prefill_tile_rows: bad dimension");
+  const int g = Hq / Hc;
+  if (g != 1 && g != 2 && g != 4 && g != 8)
+    return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill_tile_rows: Hq/Hc = %d (supported: 1, 2, 4, 8)", g);
+  if (dtype != FP_DTYPE_BF16 && dtype != FP_DTYPE_F16 && dtype != FP_DTYPE_F32)
+    return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill_tile_rows: unknown dtype %d", dtype);
+  return tile_rows_for(Lq, Hq, Hc, D, dtype, workspace_bytes);
+}
+
+extern "C" int fp_paged_prefill_tile_order(const int64_t* batch_idx, const int32_t* row_limit, int32_t Lq,
+                                           int32_t tile_rows, int32_t* order, void* stream) {
+  if (Lq < 0) return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_prefill_tile_order: negative length");
+  if (tile_rows != 32 && tile_rows != 64 && tile_rows != 128 && tile_rows != 256)
+    return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_prefill_tile_order: tile_rows = %d (32, 64, 128 or 256: ask "
+                    "fp_paged_prefill_tile_rows)", tile_rows);
+  if (Lq == 0) return FP_OK;
+  if (!batch_idx || !row_limit || !order) return fp::fail(FP_ERR_INVALID_ARGUMENT, "fp_paged_prefill_tile_order: null pointer");
+  const int n_tiles = (Lq + tile_rows - 1) / tile_rows;
+  if (n_tiles > kOrderMaxTiles)
+    return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill_tile_order: %d query tiles (at most %d)", n_tiles, kOrderMaxTiles);
+  int shift = 5;
+  while ((1 << shift) < tile_rows) ++shift;
+  hipLaunchKernelGGL(prefill_tile_order_kernel, dim3(1), dim3(kOrderThreads), 0, static_cast<hipStream_t>(stream), batch_idx,
+                     row_limit, Lq, shift, n_tiles, order);
+  return fp::check_launch("fp_paged_prefill_tile_order");
+}
 
 extern "C" int fp_paged_prefill(const void* q, int64_t q_stride_row, int64_t q_stride_h, const void* pool_k,
                                 const void* pool_v, const int64_t* page_table, int64_t pt_row_stride,
@@ -848,7 +953,8 @@ extern "C" int fp_paged_prefill(const void* q, int64_t q_stride_row, int64_t q_s
                                 int32_t Lq, int32_t Hq,
                                 int32_t Hc, int32_t D, int32_t page_size, int32_t n_pages, int32_t max_batch,
                                 int64_t n_slots, float scale, float score_bound, int dtype, void* workspace,
-                                int64_t workspace_bytes, void* stream) {
+                                int64_t workspace_bytes, const int32_t* tile_order, int32_t tile_order_rows,
+                                void* stream) {
   if (dtype != FP_DTYPE_BF16 && dtype != FP_DTYPE_F16 && dtype != FP_DTYPE_F32)
     return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill: unknown dtype %d", dtype);
   if (D != 64 && D != 128) return fp::fail(FP_ERR_UNSUPPORTED, "fp_paged_prefill: head_dim %d (supported: 64, 128)", D);
@@ -884,7 +990,8 @@ extern "C" int fp_paged_prefill(const void* q, int64_t q_stride_row, int64_t q_s
                 static_cast<const char*>(pool_k), static_cast<const char*>(pool_v),
                 page_table, pt_row_stride, batch_idx, row_limit,
                 static_cast<char*>(out), out_stride_row * 2, out_stride_h * 2, lse, sinks,
-                Lq, Hq, Hc, fp::PageDiv(page_size), n_pages, max_batch, n_slots, scale * kLog2e, 0, nullptr, nullptr};
+                Lq, Hq, Hc, fp::PageDiv(page_size), n_pages, max_batch, n_slots, scale * kLog2e, 0, nullptr, nullptr,
+                tile_order, tile_order ? tile_order_rows : 0};
   hipStream_t st = static_cast<hipStream_t>(stream);
   int rc;
   if (dtype == FP_DTYPE_BF16)

@@ -15,7 +15,7 @@ import torch
 _LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib")
 LIB_PATH = os.path.join(_LIB_DIR, "libfp_paged_kv.so")
 
-FP_ABI_VERSION = 6
+FP_ABI_VERSION = 7
 NOALLOC_SCRATCH_BYTES = 64 << 20  # FP_NOALLOC_SCRATCH_BYTES
 FP_DTYPE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
 FP_INDEX = {torch.int32: 0, torch.int64: 1}
@@ -66,7 +66,9 @@ SIGNATURES = {
         c_void_p, c_int64, c_void_p, c_void_p,
         c_void_p, c_int64, c_int64, c_void_p, c_void_p,
         c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
-        c_int64, c_float, c_float, c_int, c_void_p, c_int64, c_void_p]),
+        c_int64, c_float, c_float, c_int, c_void_p, c_int64, c_void_p, c_int32, c_void_p]),
+    "fp_paged_prefill_tile_rows": (c_int32, [c_int32, c_int32, c_int32, c_int32, c_int, c_int64]),
+    "fp_paged_prefill_tile_order": (c_int, [c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_void_p]),
     "fp_paged_prefill_workspace_bytes": (c_int64, [c_int32, c_int32, c_int32, c_int32, c_int]),
 }
 

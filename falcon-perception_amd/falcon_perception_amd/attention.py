@@ -131,6 +131,7 @@ class HybridPrefillMask:
         self._step_key = None  # (address, shape) of the positions whose row limits are kept below
         self._step_layer = -1  # layer that asked last: a layer id that does not grow starts a new step
         self._row_limit = None
+        self._tile_orders: dict[int, tuple[Tensor, int]] = {}  # rows per tile -> tile order of the step's limits
 
     def _limits_from_ids(self, open_spans, validate) -> Tensor:
         """Run the row-limit kernel and hand its report to the cache.
@@ -174,8 +175,17 @@ class HybridPrefillMask:
             reach = self.row_hi.to(torch.int64) - self._arange
             self._row_limit = (input_pos.reshape(-1) + reach).to(torch.int32)
             self._step_key = key
+            self._tile_orders = {}
         self._step_layer = layer_id
         return self._row_limit
+
+    def tile_order(self, batch_idx: Tensor, tile_rows: int) -> tuple[Tensor, int]:
+        """Query tiles of the step by decreasing key range (`ops.prefill_tile_order`), made by the first layer
+        that asks after `row_limit` and kept for the layers after it."""
+        hit = self._tile_orders.get(tile_rows)
+        if hit is None:
+            hit = self._tile_orders[tile_rows] = ops.prefill_tile_order(batch_idx, self._row_limit, tile_rows)
+        return hit
 
 
 # --------------------------------------------------------------------------
@@ -295,11 +305,20 @@ def compiled_flex_attn_prefill(q: Tensor, k: Tensor, v: Tensor, score_mod=None, 
     if step is None:
         raise RuntimeError("paged prefill attention called before PagedKVCache.insert_kv for this step")
     pool_k, pool_v = cache._planes[step.layer_id]
+    Lq, Hq, D = q.shape[2], q.shape[1], q.shape[3]
+    limits = block_mask.row_limit(step.input_pos, step.layer_id)
+    workspace = cache.prefill_workspace(Lq, Hq, D, pool_k.shape[0], q.dtype)
+    # At head_dim 64 several small workgroups share a CU and the order in which they start decides when the launch
+    # ends: the step's query tiles are ranked once (first layer) and every layer starts the longest first.  At
+    # head_dim 128 the order measured no difference, so no kernel is spent on it.
+    order = None
+    if D == 64:
+        rows = cache.prefill_tile_rows(Lq, Hq, D, pool_k.shape[0], q.dtype, workspace.numel() if workspace is not False else 0)
+        if rows and -(-Lq // rows) <= 4096:
+            order = block_mask.tile_order(step.batch_idx, rows)
     out, lse = ops.paged_prefill(
-        q, pool_k, pool_v, cache.page_table, step.batch_idx,
-        block_mask.row_limit(step.input_pos, step.layer_id), cache.page_size, scale=scale, sinks=sinks,
-        workspace=cache.prefill_workspace(q.shape[2], q.shape[1], q.shape[3], pool_k.shape[0], q.dtype),
-        score_bound=cache.score_bound(q.shape[3], scale),
+        q, pool_k, pool_v, cache.page_table, step.batch_idx, limits, cache.page_size, scale=scale, sinks=sinks,
+        workspace=workspace, score_bound=cache.score_bound(D, scale), tile_order=order,
     )
     return _result(out, lse, return_aux, return_lse)
 

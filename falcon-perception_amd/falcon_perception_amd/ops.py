@@ -348,14 +348,16 @@ def paged_prefill(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor,
                   row_limit: Tensor, page_size: int, *, scale: float | None = None,
                   out: Tensor | None = None, lse: Tensor | None = None,
                   sinks: Tensor | None = None, workspace: Tensor | None | bool = None,
-                  score_bound: float = 0.0) -> tuple[Tensor, Tensor]:
+                  score_bound: float = 0.0, tile_order: tuple[Tensor, int] | None = None) -> tuple[Tensor, Tensor]:
     """Chunked-prefill attention over the paged cache.  q [1, Hq, Lq, D]; row r sees keys
     0..row_limit[r]-1 of sequence batch_idx[r]; returns out like q, lse [1, Hq, Lq].
     `sinks` [Hq] float32 gates the output as in `paged_decode`.  `workspace`: a uint8 tensor of
     `prefill_workspace_bytes(...)` bytes lets a launch too small for the GPU be cut along the keys as
     well; None allocates one when the shape calls for it, False runs without.  `score_bound` > 0 is the
     caller's guarantee that |scale * q.k| never exceeds it (sqrt(D) for the model's normalised q and k): the
-    bf16 kernel then runs its softmax without a running maximum."""
+    bf16 kernel then runs its softmax without a running maximum.  `tile_order`: what `prefill_tile_order` returned
+    for this step (order tensor, rows per tile): the launch's workgroups then run from the longest key range to
+    the shortest; same results, faster where several small workgroups share a CU (head_dim 64)."""
     N.require_cuda(q, pool_k, pool_v, page_table, batch_idx, row_limit, out, lse)
     one, Hq, Lq, D = q.shape
     if one != 1:
@@ -389,14 +391,46 @@ def paged_prefill(q: Tensor, pool_k: Tensor, pool_v: Tensor, page_table: Tensor,
         if workspace.dtype != torch.uint8 or not workspace.is_contiguous():
             raise RuntimeError("workspace must be a contiguous uint8 tensor")
         ws_ptr, ws_bytes = workspace.data_ptr(), workspace.numel()
+    order_ptr, order_rows = None, 0
+    if tile_order is not None:
+        order, order_rows = tile_order
+        N.require_cuda(order)
+        if order.dtype != torch.int32 or not order.is_contiguous() or order.numel() != -(-Lq // order_rows):
+            raise RuntimeError("tile_order must be what prefill_tile_order returned for this step: int32, one entry per "
+                               f"tile of {order_rows} rows")
+        order_ptr = order.data_ptr()
     rc = N.lib().fp_paged_prefill(
         q.data_ptr(), q.stride(2), q.stride(1), pool_k.data_ptr(), pool_v.data_ptr(),
         page_table.data_ptr(), page_table.stride(0), batch_idx.data_ptr(),
         row_limit.data_ptr(), out.data_ptr(), out.stride(2), out.stride(1), lse.data_ptr(),
         _sinks_ptr(sinks, Hq, q.device), Lq, Hq, Hc, D, page_size, page_table.shape[1], page_table.shape[0], n_slots,
-        scale, float(score_bound), N.dtype_code(q.dtype), ws_ptr, ws_bytes, N.stream_ptr(q.device))
+        scale, float(score_bound), N.dtype_code(q.dtype), ws_ptr, ws_bytes, order_ptr, order_rows, N.stream_ptr(q.device))
     N.check(rc, "fp_paged_prefill")
     return out, lse
+
+
+def prefill_tile_rows(Lq: int, Hq: int, Hc: int, D: int, dtype: torch.dtype, workspace_bytes: int = 0) -> int:
+    """Rows per query tile of the launch `paged_prefill` makes for this shape with a workspace of this size
+    (0: the launch takes no tile order)."""
+    n = int(N.lib().fp_paged_prefill_tile_rows(Lq, Hq, Hc, D, N.dtype_code(dtype), workspace_bytes))
+    N.check(n, "fp_paged_prefill_tile_rows")
+    return n
+
+
+def prefill_tile_order(batch_idx: Tensor, row_limit: Tensor, tile_rows: int) -> tuple[Tensor, int]:
+    """The query tiles of a prefill step (tiles of `tile_rows` rows, `prefill_tile_rows`) by decreasing key range,
+    as `(order, tile_rows)` for `paged_prefill(tile_order=)`.  Once per step: every layer's launch takes the same."""
+    N.require_cuda(batch_idx, row_limit)
+    batch_idx, row_limit = batch_idx.reshape(-1), row_limit.reshape(-1)
+    if batch_idx.dtype != torch.int64 or row_limit.dtype != torch.int32 or batch_idx.numel() != row_limit.numel():
+        raise RuntimeError("batch_idx must be int64 and row_limit int32, one entry per query row each")
+    batch_idx, row_limit = batch_idx.contiguous(), row_limit.contiguous()
+    Lq = row_limit.numel()
+    order = torch.empty(-(-Lq // tile_rows) if tile_rows > 0 else 0, dtype=torch.int32, device=row_limit.device)
+    rc = N.lib().fp_paged_prefill_tile_order(batch_idx.data_ptr(), row_limit.data_ptr(), Lq, tile_rows, order.data_ptr(),
+                                             N.stream_ptr(row_limit.device))
+    N.check(rc, "fp_paged_prefill_tile_order")
+    return order, tile_rows
 
 
 def prefill_workspace_bytes(Lq: int, Hq: int, Hc: int, D: int, dtype: torch.dtype) -> int:

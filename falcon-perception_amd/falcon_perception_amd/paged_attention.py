@@ -126,6 +126,7 @@ class PagedKVCache(KVCacheBase):
         self._decode_plan_owner = None           # the mask object it was made for
         self._prefill_workspace: Tensor | None = None
         self._prefill_need: dict[tuple, int] = {}
+        self._prefill_tile_rows: dict[tuple, int] = {}
         # status word of the last prefill mask, on its way to the host (`check_prefill_masks`)
         self._mask_status_host: Tensor | None = None
         self._mask_status_event = None
@@ -507,6 +508,14 @@ class PagedKVCache(KVCacheBase):
         if not self.qk_normalised:
             return 0.0
         return 1.1 * head_dim * (head_dim ** -0.5 if scale is None else abs(scale))
+
+    def prefill_tile_rows(self, Lq: int, Hq: int, D: int, Hc: int, dtype: torch.dtype, workspace_bytes: int) -> int:
+        """Rows per query tile of the prefill launch of this shape (`ops.prefill_tile_rows`), asked once per shape."""
+        key = (Lq, Hq, Hc, D, dtype, workspace_bytes)
+        hit = self._prefill_tile_rows.get(key)
+        if hit is None:
+            hit = self._prefill_tile_rows[key] = ops.prefill_tile_rows(Lq, Hq, Hc, D, dtype, workspace_bytes)
+        return hit
 
     def prefill_workspace(self, Lq: int, Hq: int, D: int, Hc: int, dtype: torch.dtype):
         """Scratch with which the prefill kernel cuts a small launch along the keys as well, owned by the
